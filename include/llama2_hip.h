@@ -1,0 +1,281 @@
+/*
+ * llama2_hip.h -- C ABI of libllama2_hip.so, the MI355X (gfx950) implementation
+ * of ManagedLlama2's quantized batch-1 decode path.
+ *
+ * The library takes the place of ManagedCuda + the embedded PTX modules
+ * underneath the reference's C# module classes: every entry point below names
+ * the reference interface it replaces (paths relative to the reference
+ * checkout).  Kernel entry points keep the argument order of the reference's
+ * `extern "C" __global__` prototypes (the native/<kernel>.cuh headers); what the reference
+ * encoded in the launch grid (number of heads / rows) is an explicit trailing
+ * int here, because grid and block shapes are chosen inside the library.
+ *
+ * Conventions
+ *   - plain C, no C++ or framework types in any signature;
+ *   - every function returns 0 (LLAMA2_OK) on success, a negative LLAMA2_ERR_*
+ *     for rejected arguments / state, or a positive hipError_t value when the
+ *     HIP runtime failed; llama2_last_error() describes the last failure of
+ *     the calling thread;
+ *   - `llama2_half` is IEEE binary16 storage (C# System.Half, CUDA half);
+ *   - all pointers named out/x/q/... are DEVICE pointers obtained from
+ *     llama2_malloc (or any hipMalloc'ed memory of the same device);
+ *   - kernels are enqueued asynchronously on one library-owned stream, in
+ *     call order; llama2_memcpy_d2h and llama2_sync wait for them.  Like the
+ *     reference (single NULL stream, one host thread) the library is not
+ *     re-entrant.
+ */
+#ifndef LLAMA2_HIP_H
+#define LLAMA2_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#pragma GCC visibility push(default)
+#endif
+
+typedef uint16_t llama2_half;
+
+#define LLAMA2_OK 0
+#define LLAMA2_ERR_INVALID_ARGUMENT (-1) /* null / misaligned pointer, bad size, aliasing */
+#define LLAMA2_ERR_NOT_INITIALIZED (-2)  /* llama2_init not called                        */
+#define LLAMA2_ERR_UNSUPPORTED (-3)      /* shape outside what the kernels implement      */
+#define LLAMA2_ERR_NO_DEVICE (-4)        /* no usable gfx950 device                        */
+
+/* Largest softmax row, as in the reference (native/softmax_kernel.cu:5). */
+#define LLAMA2_MAX_SOFTMAX_SIZE 8192
+
+/* ---------------------------------------------------------------- runtime */
+
+/* new CudaContext(deviceID): src/Transformer.cs:48-49.  Idempotent per device. */
+int llama2_init(int device);
+/* Releases the stream and internal scratch.  Caller-owned buffers stay valid. */
+int llama2_shutdown(void);
+/* Text of the calling thread's last error ("" if none).  Never NULL. */
+const char* llama2_last_error(void);
+
+/* new CudaDeviceVariable<T>(n): src/RunState.cs:41-53.  256-byte aligned. */
+int llama2_malloc(void** ptr, size_t bytes);
+/* CudaDeviceVariable.Dispose. */
+int llama2_free(void* ptr);
+/* implicit T[] -> CudaDeviceVariable<T> (src/TransformerWeights.cs:61-66) and
+ * CopyToDevice(src, 0, dstByteOffset, bytes) (src/Extensions.cs:23-24,
+ * src/Transformer.cs:93,127).  Ordered after previously enqueued kernels. */
+int llama2_memcpy_h2d(void* dst, size_t dst_offset_bytes, const void* src, size_t bytes);
+/* explicit CudaDeviceVariable<T> -> T[] and the 1-element indexer read
+ * `runstate.tokens[nextPosition]` (src/Sampler.cs:69).  Waits for the stream. */
+int llama2_memcpy_d2h(void* dst, const void* src, size_t src_offset_bytes, size_t bytes);
+/* Asynchronous fill (tests and RunState set-up; ManagedCuda's Memset). */
+int llama2_memset(void* dst, int byte_value, size_t bytes);
+/* CudaContext.GetFreeDeviceMemorySize(): src/RunState.cs:34. */
+int llama2_mem_info(size_t* free_bytes, size_t* total_bytes);
+/* CudaContext.Synchronize(). */
+int llama2_sync(void);
+/* The hipStream_t every entry point launches on (for callers that time or
+ * order their own work against it).  NULL before llama2_init. */
+void* llama2_stream(void);
+
+/* HIP events on the library's stream, for timing the enqueued kernels. */
+int llama2_event_create(void** event);
+int llama2_event_record(void* event);
+int llama2_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
+int llama2_event_destroy(void* event);
+
+/* ------------------------------------------------- int4 tensors ("QWeight")
+ * Layout per output row n of a K-input tensor (src/TransformerWeights.cs:54-69,
+ * native/mat_vec_kernel.cu:98-134):
+ *   weights_size = ceil(K/32)*4 uint32, element k in bits 4*(k%8).. of word k/8
+ *   scales_size  = ceil(K/128)   fp16,  scale of group g = k/128
+ *   zeros_size   = ceil(scales_size/8) uint32, zero of group g = nibble g%8 of word g/8
+ *   value(n,k)   = (w - z) * scale
+ * `rows` is the INPUT length K and `cols` the number of outputs N, as in the
+ * reference (src/MatVecResidual.cs:15-22).  The three *_size arguments must be
+ * the values above (they are what the reference's modules pass); weight rows
+ * must be 16-byte aligned.
+ */
+
+/* mat_vec_residual_int4_kernel (native/mat_vec_kernel.cuh:58-59), module
+ * MatVecResidual.Forward (src/MatVecResidual.cs:15-22):
+ *   output[n] = half(float(output[n]) + sum_k input[k]*(w-z)*s).
+ * `output` must not overlap `input`. */
+int llama2_mat_vec_residual_int4(llama2_half* output, const llama2_half* input,
+                                 const uint32_t* weights, const uint32_t* zeros,
+                                 const llama2_half* scales, int rows, int cols, int zeros_size,
+                                 int scales_size, int weights_size);
+
+/* The same dot product without the residual read (device function
+ * mat_vec_int4, native/mat_vec_kernel.cu:166-177; one third of QKVMatVec). */
+int llama2_mat_vec_int4(llama2_half* output, const llama2_half* input, const uint32_t* weights,
+                        const uint32_t* zeros, const llama2_half* scales, int rows, int cols,
+                        int zeros_size, int scales_size, int weights_size);
+
+/* qkv_mat_vec_kernel (native/mat_vec_kernel.cuh:85-89), module QKVMatVec.Forward
+ * (src/QKVMatVec.cs:19-31): three int4 mat-vecs of one input in one launch.
+ * k_output / v_output are the KV-cache rows, i.e. the caller has already added
+ * layerOffset + pos*kvDim (src/QKVMatVec.cs:25-26). */
+int llama2_qkv_mat_vec(llama2_half* q_output, llama2_half* k_output, llama2_half* v_output,
+                       const llama2_half* input, const uint32_t* q_weight, const uint32_t* q_zeros,
+                       const llama2_half* q_scales, const uint32_t* k_weight,
+                       const uint32_t* k_zeros, const llama2_half* k_scales,
+                       const uint32_t* v_weight, const uint32_t* v_zeros,
+                       const llama2_half* v_scales, int rows, int cols, int zeros_size,
+                       int scales_size, int weights_size);
+
+/* mat_vec_swiglu_kernel (native/mat_vec_kernel.cuh:113-116), module
+ * MatVecSwiGLU.Forward (src/MatVecSwiGLU.cs:15-24):
+ *   output[n] = half( silu(g.x) * (u.x) ),  silu(v) = v / (1 + expf(-v)). */
+int llama2_mat_vec_swiglu(llama2_half* output, const llama2_half* input, const uint32_t* g_weight,
+                          const uint32_t* g_zeros, const llama2_half* g_scales,
+                          const uint32_t* u_weight, const uint32_t* u_zeros,
+                          const llama2_half* u_scales, int rows, int cols, int zeros_size,
+                          int scales_size, int weights_size);
+
+/* ---------------------------------------------------------- fp16 mat-vecs */
+
+/* mat_vec_kernel (native/mat_vec_kernel.cuh:17), module MatVec.Forward
+ * (src/MatVec.cs:15-16): output[n] = sum_k matrix[n*rows + k] * vector[k];
+ * rows % 8 == 0 as in the reference (native/mat_vec_kernel.cu:16,26). */
+int llama2_mat_vec(llama2_half* output, const llama2_half* vector, const llama2_half* matrix,
+                   int rows, int cols);
+
+/* mat_vec_strided_kernel (native/mat_vec_kernel.cuh:37-38), module
+ * MatVecStrided.Forward (src/MatVecStrided.cs:16-18); n_heads was gridDim.y:
+ *   output[h*o_stride + t] = alpha * sum_{r<rows} vector[h*v_stride + r]
+ *                                    * matrix[t*m_row_stride + h*m_col_stride + r]
+ * for t < cols, h < n_heads. */
+int llama2_mat_vec_strided(llama2_half* output, const llama2_half* vector,
+                           const llama2_half* matrix, int rows, int cols, int v_stride,
+                           int m_col_stride, int m_row_stride, int o_stride, float alpha,
+                           int n_heads);
+
+/* vec_mat_kernel (native/vec_mat_kernel.cuh:5-6), module VecMat.Forward
+ * (src/VecMat.cs:17-19); n_heads was gridDim.y:
+ *   output[h*o_stride + r] = sum_{t<cols} vector[h*cols + t]
+ *                            * matrix[t*m_row_stride + h*m_col_stride + r],  r < rows. */
+int llama2_vec_mat(llama2_half* output, const llama2_half* vector, const llama2_half* matrix,
+                   int rows, int cols, int m_col_stride, int o_stride, int m_row_stride,
+                   int n_heads);
+
+/* ------------------------------------------------------- pointwise modules */
+
+/* rmsnorm_kernel (native/rmsnorm_kernel.cuh:5), module RMSNorm.Forward
+ * (src/RMSNorm.cs:13-14): output[i] = half(1/sqrtf(mean(x^2)+eps) * gamma[i] * x[i]).
+ * output may be the same buffer as input (src/Transformer.cs:187). */
+int llama2_rmsnorm(llama2_half* output, const llama2_half* input, const llama2_half* gamma,
+                   int size, float eps);
+
+/* rope_kernel (native/rope_kernel.cuh:6), module RoPERotation.Forward
+ * (src/RoPERotation.cs:19-24); n_heads was gridDim.x.  Rotates the pairs
+ * (i, i + head_size/2) of every head of q, and of k for heads < n_kv_heads;
+ * k is the cache row, already offset by layerOffset + pos*kvDim. */
+int llama2_rope(llama2_half* q, llama2_half* k, int n_kv_heads, int head_size, int pos,
+                float theta, int n_heads);
+
+/* softmax_kernel (native/softmax_kernel.cuh:5), module Softmax.Forward
+ * (src/Softmax.cs:13-14); n_rows was gridDim.x: in-place softmax of
+ * vector[r*size .. r*size+size) for r < n_rows; size <= LLAMA2_MAX_SOFTMAX_SIZE. */
+int llama2_softmax(llama2_half* vector, int size, int n_rows);
+
+/* argmax_kernel (native/argmax_kernel.cuh:5), module Argmax.Forward
+ * (src/Argmax.cs:13-14): result[pos] = index of the largest input iff
+ * write_token.  Ties resolve to the LOWEST index, deterministically (the
+ * reference's CPU check, test/ArgmaxTests.cs:33-46; its kernel races). */
+int llama2_argmax(const llama2_half* input, int size, int* result, int pos, int write_token);
+
+/* embedding_kernel (native/embedding_kernel.cuh:5), module Embedding.Forward
+ * (src/Embedding.cs:13-14): output[i] = table[tokens[pos]*size + i]; the token
+ * id is read on the device. */
+int llama2_embedding(llama2_half* output, const llama2_half* table, int size, const int* tokens,
+                     int pos);
+
+/* ------------------------------------------------------------ decode step */
+
+/* src/Config.cs:6-19 -- the 32-byte model-file header, same field order. */
+typedef struct llama2_config {
+    int dim;
+    int hidden_dim;
+    int n_layers;
+    int n_heads;
+    int n_kv_heads;
+    int vocab_size;
+    int seq_len;
+    float rope_theta;
+} llama2_config;
+
+/* src/QWeight.cs:5-10 */
+typedef struct llama2_qweight {
+    const uint32_t* weight;
+    const uint32_t* zeros;
+    const llama2_half* scales;
+} llama2_qweight;
+
+/* src/PerLayerWeight.cs:5-16 */
+typedef struct llama2_layer_weights {
+    llama2_qweight query, key, value, output, gate, up, down;
+    const llama2_half* rms_attention;
+    const llama2_half* rms_feed_forward;
+} llama2_layer_weights;
+
+/* src/TransformerWeights.cs:8-14 */
+typedef struct llama2_transformer_weights {
+    const llama2_half* token_embedding_table;
+    const llama2_half* classifier_weights;
+    const llama2_half* rms_final_weight;
+    const llama2_layer_weights* layers; /* host array of n_layers entries */
+} llama2_transformer_weights;
+
+/* src/RunState.cs:7-25.  attention holds n_heads*max(dim, seq_len) halfs,
+ * key/value caches n_layers*seq_len*kv_dim halfs, tokens seq_len+1 ints. */
+typedef struct llama2_run_state {
+    llama2_half* x;
+    llama2_half* xb;
+    llama2_half* h;
+    llama2_half* q;
+    llama2_half* attention;
+    llama2_half* logits;
+    llama2_half* key_cache;
+    llama2_half* value_cache;
+    int* tokens;
+} llama2_run_state;
+
+typedef struct llama2_decoder llama2_decoder;
+
+/* How llama2_decode_forward issues the step. */
+#define LLAMA2_DECODE_MODULES 0 /* the 10 module launches per layer of Transformer.Forward */
+#define LLAMA2_DECODE_FUSED 1   /* fused kernels (norm+QKV+RoPE, attention, norm+SwiGLU, ...) */
+#define LLAMA2_DECODE_GRAPH 2   /* OR-able: replay the step as a captured hipGraph          */
+
+/* Binds a config, a weight set and a run state (all borrowed, all must outlive
+ * the decoder) to the per-step launch sequence of Transformer.Forward
+ * (src/Transformer.cs:158-190).  GQA is rejected like the reference does
+ * (src/Transformer.cs:53-56). */
+int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
+                         const llama2_transformer_weights* weights,
+                         const llama2_run_state* state, int mode);
+/* Transformer.Forward(position, nextPosition): leaves fp16 logits in
+ * state->logits.  Asynchronous. */
+int llama2_decode_forward(llama2_decoder* decoder, int position, int next_position);
+/* Sampler.Sample greedy branch (src/Sampler.cs:44-47,69): argmax into
+ * tokens[next_position] iff generate_token, then reads that token back
+ * (the one host synchronisation per token). */
+int llama2_decode_sample(llama2_decoder* decoder, int next_position, int generate_token,
+                         int* token);
+/* `steps` iterations of forward + greedy sample starting at `position`
+ * without any host synchronisation in between (tokens stay on the device;
+ * positions below n_prompt keep their prompt token, as Transformer.Generate
+ * does, src/Transformer.cs:96-104).  Does not stop on token < 3. */
+int llama2_decode_run(llama2_decoder* decoder, int position, int steps, int n_prompt);
+int llama2_decode_destroy(llama2_decoder* decoder);
+
+#if defined(__GNUC__)
+#pragma GCC visibility pop
+#endif
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLAMA2_HIP_H */

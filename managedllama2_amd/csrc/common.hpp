@@ -1,0 +1,135 @@
+// Shared host/device helpers of libllama2_hip.so (gfx950 only).
+#pragma once
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstddef>
+#include <cstdint>
+
+#include "../../include/llama2_hip.h"
+
+namespace l2 {
+
+// ------------------------------------------------------------------ host side
+struct Context {
+    bool ready = false;
+    int device = -1;
+    hipStream_t stream = nullptr;
+    int num_cus = 0;
+    // fp32 partial sums of the sequence-split attention kernels
+    float* attn_partials = nullptr;
+    size_t attn_partials_bytes = 0;
+};
+
+Context& ctx();
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char* what);
+int ensure_attn_partials(size_t bytes);
+
+#define L2_REQUIRE_INIT()                                                          \
+    do {                                                                           \
+        if (!::l2::ctx().ready)                                                    \
+            return ::l2::fail(LLAMA2_ERR_NOT_INITIALIZED, "%s: llama2_init has not been called", __func__); \
+    } while (0)
+
+#define L2_CHECK(cond, ...)                                                        \
+    do {                                                                           \
+        if (!(cond))                                                               \
+            return ::l2::fail(LLAMA2_ERR_INVALID_ARGUMENT, __VA_ARGS__);           \
+    } while (0)
+
+#define L2_HIP(expr)                                                               \
+    do {                                                                           \
+        hipError_t e_ = (expr);                                                    \
+        if (e_ != hipSuccess)                                                      \
+            return ::l2::hip_fail(e_, #expr);                                      \
+    } while (0)
+
+#define L2_LAUNCH_CHECK(name)                                                      \
+    do {                                                                           \
+        hipError_t e_ = hipGetLastError();                                         \
+        if (e_ != hipSuccess)                                                      \
+            return ::l2::hip_fail(e_, name);                                       \
+    } while (0)
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+inline bool overlap(const void* a, size_t na, const void* b, size_t nb)
+{
+    auto pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+    return pa < pb + nb && pb < pa + na;
+}
+
+// ---------------------------------------------------------------- device side
+#if defined(__HIPCC__)
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ h2_t as_h2(uint32_t v) { return __builtin_bit_cast(h2_t, v); }
+__device__ __forceinline__ uint32_t as_u32(h2_t v) { return __builtin_bit_cast(uint32_t, v); }
+
+// fp32 += a.x*b.x + a.y*b.y  (v_dot2_f32_f16: fp16 products, fp32 accumulate)
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float acc)
+{
+    return __builtin_amdgcn_fdot2(as_h2(a), as_h2(b), acc, false);
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint16_t h)
+{
+    return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+__device__ __forceinline__ uint16_t float_to_half_bits(float f)
+{
+    return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); // v_cvt_f16_f32, RNE
+}
+
+// DPP controls (GCN3/CDNA encoding)
+constexpr int DPP_QUAD_XOR1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141; // lane i <- lane 7-i within 8
+constexpr int DPP_ROW_MIRROR = 0x140;      // lane i <- lane 15-i within 16
+constexpr int DPP_ROW_BCAST15 = 0x142;     // lane 15 of each row -> next row
+constexpr int DPP_ROW_BCAST31 = 0x143;     // lane 31 -> rows 2,3
+
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_f32(float v)
+{
+    // lanes whose row is masked out (or whose source is invalid) read 0
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+
+// Sum over each 16-lane row; every lane of the row ends with the row total.
+__device__ __forceinline__ float row16_sum(float v)
+{
+    v += dpp_f32<DPP_QUAD_XOR1>(v);
+    v += dpp_f32<DPP_QUAD_XOR2>(v);
+    v += dpp_f32<DPP_ROW_HALF_MIRROR>(v);
+    v += dpp_f32<DPP_ROW_MIRROR>(v);
+    return v;
+}
+
+// Sum over the 64-lane wavefront, returned in every lane (as a scalar).
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v = row16_sum(v);
+    v += dpp_f32<DPP_ROW_BCAST15, 0xA>(v);
+    v += dpp_f32<DPP_ROW_BCAST31, 0xC>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
+__device__ __forceinline__ float wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1)
+        v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+#endif // __HIPCC__
+
+} // namespace l2

@@ -1,0 +1,227 @@
+// Runtime half of the C ABI: device context, memory, stream, events, errors.
+// Replaces what the reference gets from ManagedCuda (CudaContext,
+// CudaDeviceVariable<T>; src/Module.cs:7-26, src/RunState.cs:27-53).
+#include "common.hpp"
+
+#include <cstdio>
+#include <cstring>
+
+namespace l2 {
+
+static Context g_ctx;
+static thread_local char g_err[512] = "";
+
+Context& ctx() { return g_ctx; }
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what)
+{
+    snprintf(g_err, sizeof(g_err), "%s: %s (%d)", what, hipGetErrorString(e), static_cast<int>(e));
+    return static_cast<int>(e);
+}
+
+int ensure_attn_partials(size_t bytes)
+{
+    Context& c = ctx();
+    if (bytes <= c.attn_partials_bytes)
+        return LLAMA2_OK;
+    // Grow only between launches that use it: earlier kernels on the stream may
+    // still read the old buffer, so drain the stream first.
+    L2_HIP(hipStreamSynchronize(c.stream));
+    if (c.attn_partials)
+        L2_HIP(hipFree(c.attn_partials));
+    c.attn_partials = nullptr;
+    c.attn_partials_bytes = 0;
+    L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.attn_partials), bytes));
+    c.attn_partials_bytes = bytes;
+    return LLAMA2_OK;
+}
+
+} // namespace l2
+
+using namespace l2;
+
+extern "C" {
+
+const char* llama2_last_error(void) { return g_err; }
+
+int llama2_init(int device)
+{
+    Context& c = ctx();
+    if (c.ready && c.device == device)
+        return LLAMA2_OK;
+    if (c.ready)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_init: already bound to device %d", c.device);
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0)
+        return fail(LLAMA2_ERR_NO_DEVICE, "llama2_init: no HIP device (%s)", hipGetErrorString(e));
+    if (device < 0 || device >= count)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_init: device %d out of range [0,%d)", device, count);
+    L2_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    L2_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(LLAMA2_ERR_NO_DEVICE, "llama2_init: device %d is %s, this library is built for gfx950 only",
+                    device, prop.gcnArchName);
+    c.num_cus = prop.multiProcessorCount;
+    L2_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+    c.device = device;
+    c.ready = true;
+    g_err[0] = 0;
+    return LLAMA2_OK;
+}
+
+int llama2_shutdown(void)
+{
+    Context& c = ctx();
+    if (!c.ready)
+        return LLAMA2_OK;
+    L2_HIP(hipStreamSynchronize(c.stream));
+    if (c.attn_partials)
+        L2_HIP(hipFree(c.attn_partials));
+    c.attn_partials = nullptr;
+    c.attn_partials_bytes = 0;
+    L2_HIP(hipStreamDestroy(c.stream));
+    c.stream = nullptr;
+    c.ready = false;
+    c.device = -1;
+    return LLAMA2_OK;
+}
+
+int llama2_malloc(void** ptr, size_t bytes)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(ptr != nullptr, "llama2_malloc: ptr is null");
+    *ptr = nullptr;
+    L2_CHECK(bytes > 0, "llama2_malloc: zero-sized allocation");
+    L2_HIP(hipMalloc(ptr, bytes));
+    return LLAMA2_OK;
+}
+
+int llama2_free(void* ptr)
+{
+    L2_REQUIRE_INIT();
+    if (!ptr)
+        return LLAMA2_OK;
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    L2_HIP(hipFree(ptr));
+    return LLAMA2_OK;
+}
+
+int llama2_memcpy_h2d(void* dst, size_t dst_offset_bytes, const void* src, size_t bytes)
+{
+    L2_REQUIRE_INIT();
+    if (bytes == 0)
+        return LLAMA2_OK;
+    L2_CHECK(dst && src, "llama2_memcpy_h2d: null pointer");
+    // Pageable source: hipMemcpyAsync stages it before returning, so the host
+    // buffer may be reused at once, and the copy is ordered on the stream.
+    L2_HIP(hipMemcpyAsync(static_cast<char*>(dst) + dst_offset_bytes, src, bytes, hipMemcpyHostToDevice,
+                          ctx().stream));
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    return LLAMA2_OK;
+}
+
+int llama2_memcpy_d2h(void* dst, const void* src, size_t src_offset_bytes, size_t bytes)
+{
+    L2_REQUIRE_INIT();
+    if (bytes == 0)
+        return LLAMA2_OK;
+    L2_CHECK(dst && src, "llama2_memcpy_d2h: null pointer");
+    L2_HIP(hipMemcpyAsync(dst, static_cast<const char*>(src) + src_offset_bytes, bytes,
+                          hipMemcpyDeviceToHost, ctx().stream));
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    return LLAMA2_OK;
+}
+
+__global__ void fill_bytes_kernel(uint8_t* dst, uint8_t v, size_t n)
+{
+    size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+    size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+    for (; i < n; i += stride)
+        dst[i] = v;
+}
+
+int llama2_memset(void* dst, int byte_value, size_t bytes)
+{
+    L2_REQUIRE_INIT();
+    if (bytes == 0)
+        return LLAMA2_OK;
+    L2_CHECK(dst, "llama2_memset: null pointer");
+    // A fill kernel rather than hipMemsetAsync, so the call stays safe to
+    // record into a captured graph.
+    size_t blocks = (bytes + 255) / 256;
+    if (blocks > 4096)
+        blocks = 4096;
+    hipLaunchKernelGGL(fill_bytes_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx().stream,
+                       static_cast<uint8_t*>(dst), static_cast<uint8_t>(byte_value), bytes);
+    L2_LAUNCH_CHECK("fill_bytes_kernel");
+    return LLAMA2_OK;
+}
+
+int llama2_mem_info(size_t* free_bytes, size_t* total_bytes)
+{
+    L2_REQUIRE_INIT();
+    size_t f = 0, t = 0;
+    L2_HIP(hipMemGetInfo(&f, &t));
+    if (free_bytes)
+        *free_bytes = f;
+    if (total_bytes)
+        *total_bytes = t;
+    return LLAMA2_OK;
+}
+
+int llama2_sync(void)
+{
+    L2_REQUIRE_INIT();
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    return LLAMA2_OK;
+}
+
+void* llama2_stream(void) { return ctx().ready ? static_cast<void*>(ctx().stream) : nullptr; }
+
+int llama2_event_create(void** event)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(event, "llama2_event_create: null pointer");
+    hipEvent_t ev;
+    L2_HIP(hipEventCreate(&ev));
+    *event = ev;
+    return LLAMA2_OK;
+}
+
+int llama2_event_record(void* event)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(event, "llama2_event_record: null event");
+    L2_HIP(hipEventRecord(static_cast<hipEvent_t>(event), ctx().stream));
+    return LLAMA2_OK;
+}
+
+int llama2_event_elapsed_ms(void* start, void* stop, float* ms)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(start && stop && ms, "llama2_event_elapsed_ms: null pointer");
+    L2_HIP(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+    L2_HIP(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+    return LLAMA2_OK;
+}
+
+int llama2_event_destroy(void* event)
+{
+    L2_REQUIRE_INIT();
+    if (event)
+        L2_HIP(hipEventDestroy(static_cast<hipEvent_t>(event)));
+    return LLAMA2_OK;
+}
+
+} // extern "C"

@@ -23,11 +23,17 @@ def rng_for(*stream):
     return np.random.Generator(np.random.PCG64([BASE_SEED, *stream]))
 
 
+def _raw_u32(rng, n):
+    """n uniform 32-bit words straight from the bit generator (an order of
+    magnitude faster than Generator.integers for gigabytes of nibbles)."""
+    return rng.bit_generator.random_raw((n + 1) // 2).view(np.uint32)[:n].copy()
+
+
 def random_qweight(rng, K, N):
     """One int4 tensor with N output rows of K inputs -> (W, Z, S) flat arrays."""
     ws, ss, zs = qweight_sizes(K)
-    W = rng.integers(0, 1 << 32, size=N * ws, dtype=np.uint32)
-    Z = rng.integers(0, 1 << 32, size=N * zs, dtype=np.uint32)
+    W = _raw_u32(rng, N * ws)
+    Z = _raw_u32(rng, N * zs)
     S = (0.002 + 0.018 * rng.random(N * ss, dtype=np.float32)).astype(np.float16)
     return W, Z, S
 

@@ -1,0 +1,53 @@
+"""Shared helpers of the GPU parity tests: every test talks to the kernels
+through the C ABI (ctypes), the way the reference's xUnit tests talk to the
+raw kernels through ManagedCuda."""
+import numpy as np
+
+from managedllama2_amd import capi, synth
+from managedllama2_amd.device import DeviceVariable, QWeight, init
+
+TOL = 2e-3  # max relative error against the fp64 dequantise-then-dot oracle
+
+
+def up(a):
+    return DeviceVariable.from_host(a)
+
+
+def upq(q):
+    return QWeight.from_host(*q)
+
+
+def sizes(K):
+    ws, ss, zs = synth.qweight_sizes(K)
+    return zs, ss, ws
+
+
+def rel_err(y, y_ref):
+    y = np.asarray(y, np.float64)
+    y_ref = np.asarray(y_ref, np.float64)
+    floor = np.max(np.abs(y_ref)) * 2.0 ** -10
+    return np.abs(y - y_ref) / np.maximum(np.abs(y_ref), max(floor, 1e-30))
+
+
+def assert_close(y, y_ref, what="", tol=TOL):
+    e = rel_err(y, y_ref)
+    worst = int(np.argmax(e))
+    assert e[worst] <= tol, "%s: max rel err %.3e at %d (got %r want %r)" % (
+        what, e[worst], worst, np.asarray(y).ravel()[worst], np.asarray(y_ref).ravel()[worst])
+
+
+def ulp_diff(a, b):
+    """Distance in fp16 representable steps."""
+    def key(h):
+        u = h.view(np.uint16).astype(np.int32)
+        return np.where(u & 0x8000, -(u & 0x7FFF), u)
+    return np.abs(key(np.asarray(a, np.float16)) - key(np.asarray(b, np.float16)))
+
+
+def assert_close_normwise(y, y_ref, what="", tol=TOL):
+    y = np.asarray(y, np.float64)
+    y_ref = np.asarray(y_ref, np.float64)
+    e = np.abs(y - y_ref) / np.max(np.abs(y_ref))
+    worst = int(np.argmax(e))
+    assert e[worst] <= tol, "%s: max norm-wise err %.3e at %d (got %r want %r)" % (
+        what, e[worst], worst, y.ravel()[worst], y_ref.ravel()[worst])
