@@ -85,6 +85,18 @@ int llama2_event_record(void* event);
 int llama2_event_elapsed_ms(void* start, void* stop, float* ms); /* waits for `stop` */
 int llama2_event_destroy(void* event);
 
+/* Stream capture of the calls made between begin and end into a hipGraph that
+ * llama2_graph_launch replays with a single submission (no counterpart in the
+ * reference, which pays one cuLaunchKernel per module call, src/Module.cs:21-22).
+ * Only kernel entry points may be called while capturing: no malloc / free /
+ * memcpy / sync, and llama2_vec_mat only for shapes whose scratch already
+ * exists (call it once eagerly first).  The captured calls keep the argument
+ * values they were made with. */
+int llama2_graph_begin_capture(void);
+int llama2_graph_end_capture(void** graph);
+int llama2_graph_launch(void* graph);
+int llama2_graph_destroy(void* graph);
+
 /* ------------------------------------------------- int4 tensors ("QWeight")
  * Layout per output row n of a K-input tensor (src/TransformerWeights.cs:54-69,
  * native/mat_vec_kernel.cu:98-134):

@@ -74,6 +74,10 @@ _SIGNATURES = {
     "llama2_memset": [vp, i, sz],
     "llama2_mem_info": [C.POINTER(sz), C.POINTER(sz)],
     "llama2_sync": [],
+    "llama2_graph_begin_capture": [],
+    "llama2_graph_end_capture": [C.POINTER(vp)],
+    "llama2_graph_launch": [vp],
+    "llama2_graph_destroy": [vp],
     "llama2_event_create": [C.POINTER(vp)],
     "llama2_event_record": [vp],
     "llama2_event_elapsed_ms": [vp, vp, C.POINTER(f)],

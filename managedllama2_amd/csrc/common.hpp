@@ -18,6 +18,7 @@ struct Context {
     int device = -1;
     hipStream_t stream = nullptr;
     int num_cus = 0;
+    bool capturing = false; // between llama2_graph_begin_capture and _end_capture
     // fp32 partial sums of the sequence-split attention kernels
     float* attn_partials = nullptr;
     size_t attn_partials_bytes = 0;

@@ -4,24 +4,24 @@
 // Shape of the computation (batch-1 GEMV, HBM-bound, no MFMA):
 //   * a "chunk" is 16 bytes of one weight row = 4 uint32 = 32 nibbles; a
 //     64-lane wavefront reads 64 consecutive chunks (1 KiB) per load
-//     instruction, lane l taking chunk j*64+l (global_load_dwordx4);
+//     instruction, lane l taking chunks l, l+64, ... (buffer_load_dwordx4
+//     through a per-row buffer resource, so the ragged end of a row reads as
+//     zero without any lane predication);
+//   * wavefronts are persistent: each walks over its rows with the next row's
+//     loads already in flight while the current one is reduced;
 //   * the input vector is staged once per workgroup in LDS, pre-permuted to
 //     the order the nibble extraction produces, in four planes so that
 //     consecutive lanes read consecutive 16-byte slots (conflict-free
-//     ds_read_b128);
-//   * nibbles become fp16 pairs with the exponent-OR trick
-//     ((w & 0x000F000F) | 0x6400'6400 = 1024+n), the zero-point is removed
-//     exactly in fp16 (v_pk_add_f16 / v_pk_fma_f16), products are accumulated
-//     in fp32 with v_dot2_f32_f16, and each chunk's partial sum is multiplied
-//     once by its group scale in fp32;
-//   * lanes are reduced with DPP row operations, lane 63 owns the total.
+//     ds_read_b128), together with the fp32 sum of every 32-element chunk;
+//   * a nibble masked in place (w & 0x000F000F, w & 0x00F000F0) IS an fp16
+//     subnormal pair (n * 2^-24 resp. n * 2^-20): v_dot2_f32_f16 multiplies it
+//     exactly with the fp16 input pair and accumulates in fp32, so dequantising
+//     costs one v_and per pair.  The zero-point is applied per chunk as
+//     -z * sum(x), the group scale once per chunk, all in fp32;
+//   * lanes are reduced with DPP row operations.
 #include "common.hpp"
 
 namespace l2 {
-
-constexpr int kWaves = 4;                // wavefronts per workgroup
-constexpr int kThreads = kWaves * 64;    // 256
-constexpr int kMaxLdsBytes = 64 * 1024;  // static+dynamic LDS we ask for
 
 struct QW {
     const uint32_t* w;
@@ -29,192 +29,269 @@ struct QW {
     const uint16_t* s;
 };
 
-struct Frag { // what one lane holds of one row for one chunk
-    u32x4 w;
-    uint32_t zword;
-    uint16_t sbits;
+enum Mode { PLAIN = 0, RESIDUAL = 1, SWIGLU = 2 };
+
+struct Int4Args {
+    QW m[3];          // PLAIN/RESIDUAL: m[0] (QKV: q,k,v); SWIGLU: gate, up
+    uint16_t* out[3]; // one output vector per tensor (SWIGLU: out[0])
+    const uint16_t* x;
+    int K, N, ws, ss, zs;
+    int n_tensors;
 };
 
-__device__ __forceinline__ Frag load_frag(const QW& m, size_t row, int c, int ws, int ss, int zs, bool valid)
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes)
 {
-    Frag f;
-    if (valid) {
-        const int g = c >> 2;
-        f.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(m.w + row * ws) + c);
-        f.zword = m.z[row * zs + (g >> 3)];
-        f.sbits = m.s[row * ss + g];
-    } else {
-        f.w = u32x4{0u, 0u, 0u, 0u};
-        f.zword = 0u;
-        f.sbits = 0;
-    }
-    return f;
+    // raw buffer, 32-bit elements; out-of-range reads return 0
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(bytes), 0x00020000);
 }
 
-// Partial dot product of one chunk (32 elements) of one row.
-__device__ __forceinline__ float chunk_dot(const Frag& f, int c, const u32x4 (&x)[4])
+constexpr int kAuxStream = 2; // "nt": weights are touched once
+
+template <int J, int R>
+struct Frag { // what one lane holds of R rows: J chunks each + its group's zero word and scale
+    u32x4 w[R][J];
+    uint32_t zw[R][J];
+    uint16_t sb[R][J];
+};
+
+template <int J>
+__device__ __forceinline__ void load_row(u32x4 (&w)[J], uint32_t (&zw)[J], uint16_t (&sb)[J], const QW& m,
+                                         size_t row, int ws, int ss, int zs, int lane)
 {
-    const uint32_t z = (f.zword >> (((c >> 2) & 7) * 4)) & 0xFu;
-    // -(1024 + z) and -(64 + z) as fp16 pairs: ulp(1024) = 1, ulp(64) = 1/16
-    const uint32_t neg_a = 0xE400E400u + z * 0x00010001u;
-    const uint32_t neg_b = 0xD400D400u + z * 0x00100010u;
-    const h2_t sixteenth = {static_cast<_Float16>(0.0625f), static_cast<_Float16>(0.0625f)};
-    float acc0 = 0.0f, acc1 = 0.0f;
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(m.w + row * ws, ws * 4);
+    const __amdgpu_buffer_rsrc_t rz = make_rsrc(m.z + row * zs, zs * 4);
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.s + row * ss, ss * 2);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t w = f.w[i];
-        const uint32_t w8 = w >> 8;
-        // (n0,n4) (n1,n5) (n2,n6) (n3,n7), each minus the zero-point, exact in fp16
-        const h2_t a0 = as_h2((w & 0x000F000Fu) | 0x64006400u) + as_h2(neg_a);
-        const h2_t a1 = __builtin_elementwise_fma(as_h2((w & 0x00F000F0u) | 0x64006400u), sixteenth, as_h2(neg_b));
-        const h2_t a2 = as_h2((w8 & 0x000F000Fu) | 0x64006400u) + as_h2(neg_a);
-        const h2_t a3 = __builtin_elementwise_fma(as_h2((w8 & 0x00F000F0u) | 0x64006400u), sixteenth, as_h2(neg_b));
-        acc0 = __builtin_amdgcn_fdot2(a0, as_h2(x[i][0]), acc0, false);
-        acc1 = __builtin_amdgcn_fdot2(a1, as_h2(x[i][1]), acc1, false);
-        acc0 = __builtin_amdgcn_fdot2(a2, as_h2(x[i][2]), acc0, false);
-        acc1 = __builtin_amdgcn_fdot2(a3, as_h2(x[i][3]), acc1, false);
+    for (int j = 0; j < J; ++j) {
+        // chunk c = lane + 64 j: group c/4, zero word c/32
+        w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
+        zw[j] = __builtin_amdgcn_raw_buffer_load_b32(rz, (lane >> 5) * 4 + j * 8, 0, 0);
+        sb[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, (lane >> 2) * 2 + j * 32, 0, 0);
     }
-    return (acc0 + acc1) * half_bits_to_float(f.sbits);
 }
 
-// Stage the K-element input in LDS as 4 planes of nchunks 16-byte slots:
-// slot (i, c) holds elements 8*(4c+i)+{0,4,1,5,2,6,3,7}; elements >= K are 0.
-__device__ __forceinline__ void stage_input(u32x4* xs, const uint16_t* x, int K, int nchunks)
-{
-    const int nwords = nchunks * 4;
-    for (int e = threadIdx.x; e < nwords; e += kThreads) {
-        u32x4 in;
-        if (8 * e + 8 <= K) {
-            in = *reinterpret_cast<const u32x4*>(x + 8 * e);
-        } else {
-            uint16_t t[8];
+// Stage the input in LDS: xs[i*JC + c] holds elements 8*(4c+i)+{0,4,1,5,2,6,3,7}
+// (JC = 64 J chunks, zero beyond K), sx[c] the fp32 sum of chunk c.
+template <int J, int T>
+struct XStage {
+    static constexpr int JC = J * 64;
+    static constexpr int XE = (JC * 4 + T - 1) / T;
+    u32x4 in[XE];
+    __device__ __forceinline__ void issue(const uint16_t* x, int K)
+    {
+        const __amdgpu_buffer_rsrc_t rx = make_rsrc(x, K * 2);
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
-                t[i] = (8 * e + i < K) ? x[8 * e + i] : uint16_t(0);
-            in = u32x4{uint32_t(t[0]) | (uint32_t(t[1]) << 16), uint32_t(t[2]) | (uint32_t(t[3]) << 16),
-                       uint32_t(t[4]) | (uint32_t(t[5]) << 16), uint32_t(t[6]) | (uint32_t(t[7]) << 16)};
+        for (int i = 0; i < XE; ++i)
+            in[i] = __builtin_amdgcn_raw_buffer_load_b128(rx, (threadIdx.x + i * T) * 16, 0, 0);
+    }
+    __device__ __forceinline__ void commit(u32x4* xs, float* sx)
+    {
+#pragma unroll
+        for (int i = 0; i < XE; ++i) {
+            const int e = threadIdx.x + i * T;
+            if (e < JC * 4) {
+                const u32x4 v = in[i];
+                u32x4 o;
+                o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);     // x0,x4
+                o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u); // x1,x5
+                o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);     // x2,x6
+                o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u); // x3,x7
+                xs[(e & 3) * JC + (e >> 2)] = o;
+                const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+                float s = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
+                s += dpp_f32<DPP_QUAD_XOR1>(s); // the 4 words of a chunk sit in one quad
+                s += dpp_f32<DPP_QUAD_XOR2>(s);
+                if ((e & 3) == 0)
+                    sx[e >> 2] = s;
+            }
         }
-        u32x4 out;
-        out[0] = (in[0] & 0xFFFFu) | (in[2] << 16);          // x0,x4
-        out[1] = (in[0] >> 16) | (in[2] & 0xFFFF0000u);      // x1,x5
-        out[2] = (in[1] & 0xFFFFu) | (in[3] << 16);          // x2,x6
-        out[3] = (in[1] >> 16) | (in[3] & 0xFFFF0000u);      // x3,x7
-        xs[(e & 3) * nchunks + (e >> 2)] = out;
     }
-}
+};
 
-// R rows of one wavefront against the staged input; sums valid in every lane.
-template <int R>
-__device__ __forceinline__ void dot_rows(float (&sum)[R], const QW (&m)[R], const size_t (&row)[R],
-                                         const u32x4* xs, const uint16_t* x, int K, int nchunks,
-                                         int ws, int ss, int zs)
+// Dot products of R rows (J chunks per lane each) with the staged input.
+template <int J, int R>
+__device__ __forceinline__ void dot_frag(float (&acc)[R], const Frag<J, R>& f, const u32x4* xs, const float* sx,
+                                         int lane, int zshift)
 {
-    const int lane = threadIdx.x & 63;
-    Frag cur[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-        cur[r] = load_frag(m[r], row[r], lane, ws, ss, zs, lane < nchunks);
-
-    // weight loads are in flight while the input is staged
-    stage_input(const_cast<u32x4*>(xs), x, K, nchunks);
-    __syncthreads();
-
-    float acc[R];
+    constexpr int JC = J * 64;
 #pragma unroll
     for (int r = 0; r < R; ++r)
         acc[r] = 0.0f;
-
-    for (int c = lane; c < nchunks + lane; c += 64) { // uniform trip count; c < nchunks masks lanes
-        const int cn = c + 64;
-        Frag nxt[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-            nxt[r] = load_frag(m[r], row[r], cn, ws, ss, zs, cn < nchunks);
-        if (c < nchunks) {
-            u32x4 xv[4];
+    for (int j = 0; j < J; ++j) {
+        const int c = lane + 64 * j;
+        u32x4 xv[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                xv[i] = xs[i * nchunks + c];
+        for (int i = 0; i < 4; ++i)
+            xv[i] = xs[i * JC + c];
+        const float sxv = sx[c];
 #pragma unroll
-            for (int r = 0; r < R; ++r)
-                acc[r] += chunk_dot(cur[r], c, xv);
-        }
+        for (int r = 0; r < R; ++r) {
+            float a0 = 0.0f, a1 = 0.0f; // a0: nibbles at bit 0 of a byte (x 2^-24), a1: at bit 4 (x 2^-20)
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-            cur[r] = nxt[r];
-    }
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-        sum[r] = wave_sum(acc[r]);
-}
-
-struct PlainArgs {
-    QW m[3];
-    uint16_t* out[3];
-};
-
-// blockIdx.y selects the tensor (1 for plain/residual, 3 for fused QKV);
-// each wavefront owns R consecutive output rows.
-template <int R, bool RESIDUAL>
-__global__ __launch_bounds__(kThreads) void int4_matvec_kernel(PlainArgs a, const uint16_t* x, int K, int N,
-                                                               int ws, int ss, int zs)
-{
-    extern __shared__ u32x4 xs[];
-    const int nchunks = ws >> 2;
-    const QW m = a.m[blockIdx.y];
-    uint16_t* out = a.out[blockIdx.y];
-    const int wave = threadIdx.x >> 6;
-    const int n0 = (blockIdx.x * kWaves + wave) * R;
-    QW ms[R];
-    size_t rows[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        ms[r] = m;
-        rows[r] = static_cast<size_t>(n0 + r < N ? n0 + r : N - 1);
-    }
-    float sum[R];
-    dot_rows<R>(sum, ms, rows, xs, x, K, nchunks, ws, ss, zs);
-    const int lane = threadIdx.x & 63;
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        if (lane == r && n0 + r < N) {
-            float v = sum[r];
-            if (RESIDUAL)
-                v += half_bits_to_float(out[n0 + r]);
-            out[n0 + r] = float_to_half_bits(v);
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t w = f.w[r][j][i], w8 = w >> 8;
+                a0 = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[i][0]), a0, false);  // n0,n4
+                a1 = __builtin_amdgcn_fdot2(as_h2(w & 0x00F000F0u), as_h2(xv[i][1]), a1, false);  // n1,n5
+                a0 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[i][2]), a0, false); // n2,n6
+                a1 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), as_h2(xv[i][3]), a1, false); // n3,n7
+            }
+            const float zf = static_cast<float>((f.zw[r][j] >> zshift) & 0xFu);
+            float t = a0 * 16777216.0f;      // 2^24
+            t = fmaf(a1, 1048576.0f, t);     // 2^20
+            t = fmaf(-zf, sxv, t);           // sum x (n - z)
+            acc[r] = fmaf(t, half_bits_to_float(f.sb[r][j]), acc[r]);
         }
     }
 }
 
-// Each wavefront owns O outputs: rows n of the gate and of the up tensor.
-template <int O>
-__global__ __launch_bounds__(kThreads) void int4_swiglu_kernel(QW g, QW u, uint16_t* out, const uint16_t* x,
-                                                               int K, int N, int ws, int ss, int zs)
+// PLAIN / RESIDUAL: item = one output row of tensor item / N (fused QKV has 3).
+// SWIGLU: item = one output n; rows n of the gate and of the up tensor.
+template <int J, int MODE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void int4_matvec_kernel(Int4Args a)
 {
-    extern __shared__ u32x4 xs[];
-    const int nchunks = ws >> 2;
-    const int wave = threadIdx.x >> 6;
-    const int n0 = (blockIdx.x * kWaves + wave) * O;
-    QW ms[2 * O];
-    size_t rows[2 * O];
-#pragma unroll
-    for (int o = 0; o < O; ++o) {
-        const size_t n = static_cast<size_t>(n0 + o < N ? n0 + o : N - 1);
-        ms[2 * o] = g;
-        ms[2 * o + 1] = u;
-        rows[2 * o] = n;
-        rows[2 * o + 1] = n;
+    constexpr int R = MODE == SWIGLU ? 2 : 1;
+    constexpr int JC = J * 64;
+    constexpr int T = WAVES * 64;
+    __shared__ u32x4 xs[4 * JC];
+    __shared__ float sx[JC];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int total_waves = gridDim.x * WAVES;
+    const int nitems = a.n_tensors * a.N;
+    int item = blockIdx.x * WAVES + wave;
+
+    auto load_item = [&](Frag<J, R>& f, uint16_t& res, int it) {
+        it = __builtin_amdgcn_readfirstlane(it);
+        if (MODE == SWIGLU) {
+            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[0], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
+            load_row<J>(f.w[R - 1], f.zw[R - 1], f.sb[R - 1], a.m[1], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
+        } else {
+            const int t = it / a.N, n = it - t * a.N;
+            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[t], static_cast<size_t>(n), a.ws, a.ss, a.zs, lane);
+            if (MODE == RESIDUAL)
+                res = a.out[t][n];
+        }
+    };
+
+    XStage<J, T> stage;
+    stage.issue(a.x, a.K); // input first (L2), then the first item's weights (HBM)
+    Frag<J, R> cur;
+    uint16_t cur_res = 0;
+    if (item < nitems)
+        load_item(cur, cur_res, item);
+    stage.commit(xs, sx);
+    __syncthreads();
+
+    const int zshift = ((lane >> 2) & 7) * 4; // nibble of the zero word: group (c/4) % 8, same for every j
+    for (; item < nitems; item += total_waves) {
+        Frag<J, R> nxt;
+        uint16_t nxt_res = 0;
+        if (item + total_waves < nitems)
+            load_item(nxt, nxt_res, item + total_waves);
+        float acc[R];
+        dot_frag<J, R>(acc, cur, xs, sx, lane, zshift);
+        if (MODE == SWIGLU) {
+            const float g = wave_sum(acc[0]);
+            const float u = wave_sum(acc[R - 1]);
+            if (lane == 0) {
+                float v = g;
+                v *= 1.0f / (1.0f + expf(-v));
+                v *= u;
+                a.out[0][item] = float_to_half_bits(v);
+            }
+        } else {
+            float v = wave_sum(acc[0]);
+            if (lane == 0) {
+                const int t = item / a.N, n = item - t * a.N;
+                if (MODE == RESIDUAL)
+                    v += half_bits_to_float(cur_res);
+                a.out[t][n] = float_to_half_bits(v);
+            }
+        }
+        cur = nxt;
+        cur_res = nxt_res;
     }
-    float sum[2 * O];
-    dot_rows<2 * O>(sum, ms, rows, xs, x, K, nchunks, ws, ss, zs);
-    const int lane = threadIdx.x & 63;
+}
+
+// Any K (fallback beyond 8 chunk-columns per lane): runtime trip count, dynamic LDS.
+template <int MODE>
+__global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
+{
+    constexpr int R = MODE == SWIGLU ? 2 : 1;
+    extern __shared__ u32x4 xs_dyn[];
+    const int nchunks = a.ws >> 2;
+    float* sx = reinterpret_cast<float*>(xs_dyn + 4 * nchunks);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int total_waves = gridDim.x * 4;
+    const int nitems = a.n_tensors * a.N;
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, a.K * 2);
+    for (int e = threadIdx.x; e < nchunks * 4; e += 256) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rx, e * 16, 0, 0);
+        u32x4 o;
+        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);
+        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u);
+        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);
+        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u);
+        xs_dyn[(e & 3) * nchunks + (e >> 2)] = o;
+        const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+        float s = 0.0f;
 #pragma unroll
-    for (int o = 0; o < O; ++o) {
-        if (lane == o && n0 + o < N) {
-            float v = sum[2 * o];
-            v *= 1.0f / (1.0f + expf(-v));
-            v *= sum[2 * o + 1];
-            out[n0 + o] = float_to_half_bits(v);
+        for (int k = 0; k < 4; ++k)
+            s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
+        s += dpp_f32<DPP_QUAD_XOR1>(s);
+        s += dpp_f32<DPP_QUAD_XOR2>(s);
+        if ((e & 3) == 0)
+            sx[e >> 2] = s;
+    }
+    __syncthreads();
+    const int zshift = ((lane >> 2) & 7) * 4;
+    for (int item = blockIdx.x * 4 + wave; item < nitems; item += total_waves) {
+        const int it = __builtin_amdgcn_readfirstlane(item);
+        const int t = MODE == SWIGLU ? 0 : it / a.N, n = MODE == SWIGLU ? it : it - t * a.N;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const QW& m = a.m[MODE == SWIGLU ? r : t];
+            const __amdgpu_buffer_rsrc_t rw = make_rsrc(m.w + static_cast<size_t>(n) * a.ws, a.ws * 4);
+            const __amdgpu_buffer_rsrc_t rz = make_rsrc(m.z + static_cast<size_t>(n) * a.zs, a.zs * 4);
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.s + static_cast<size_t>(n) * a.ss, a.ss * 2);
+            float s = 0.0f;
+            for (int c0 = 0; c0 < nchunks; c0 += 64) {
+                const int c = c0 + lane; // beyond nchunks the buffer reads 0, the LDS index is clamped
+                const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(rw, c * 16, 0, kAuxStream);
+                const uint32_t zw = __builtin_amdgcn_raw_buffer_load_b32(rz, (c >> 5) * 4, 0, 0);
+                const uint16_t sb = __builtin_amdgcn_raw_buffer_load_b16(rs, (c >> 2) * 2, 0, 0);
+                const int cc = c < nchunks ? c : nchunks - 1;
+                float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const u32x4 xv = xs_dyn[i * nchunks + cc];
+                    const uint32_t w = w4[i], w8 = w >> 8;
+                    a0 = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[0]), a0, false);
+                    a1 = __builtin_amdgcn_fdot2(as_h2(w & 0x00F000F0u), as_h2(xv[1]), a1, false);
+                    a0 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[2]), a0, false);
+                    a1 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), as_h2(xv[3]), a1, false);
+                }
+                const float zf = static_cast<float>((zw >> zshift) & 0xFu);
+                float tt = a0 * 16777216.0f;
+                tt = fmaf(a1, 1048576.0f, tt);
+                tt = fmaf(-zf, c < nchunks ? sx[cc] : 0.0f, tt);
+                s = fmaf(tt, half_bits_to_float(sb), s);
+            }
+            acc[r] = wave_sum(s);
+        }
+        if (lane == 0) {
+            float v = acc[0];
+            if (MODE == SWIGLU) {
+                v *= 1.0f / (1.0f + expf(-v));
+                v *= acc[R - 1];
+            } else if (MODE == RESIDUAL) {
+                v += half_bits_to_float(a.out[t][n]);
+            }
+            a.out[t][n] = float_to_half_bits(v);
         }
     }
 }
@@ -228,11 +305,14 @@ static int check_qweight_call(const char* fn, const void* out, const void* in, i
     L2_CHECK(scales_size == ss && weights_size == ws && zeros_size == zs,
              "%s: sizes (zeros %d, scales %d, weights %d) do not match rows=%d (expected %d, %d, %d)", fn,
              zeros_size, scales_size, weights_size, rows, zs, ss, ws);
+    L2_CHECK(rows % 8 == 0, "%s: rows=%d must be a multiple of 8 (the input is read 16 bytes at a time, as in the reference)",
+             fn, rows);
     L2_CHECK(aligned(in, 16), "%s: input must be 16-byte aligned", fn);
     L2_CHECK(aligned(out, 2), "%s: output must be 2-byte aligned", fn);
-    if (static_cast<size_t>(ws) * 16 > static_cast<size_t>(kMaxLdsBytes))
-        return fail(LLAMA2_ERR_UNSUPPORTED, "%s: rows=%d needs %d bytes of LDS, limit %d", fn, rows, ws * 16,
-                    kMaxLdsBytes);
+    if (static_cast<size_t>(ws) * 17 > 64 * 1024)
+        return fail(LLAMA2_ERR_UNSUPPORTED, "%s: rows=%d does not fit the 64 KiB LDS staging buffer", fn, rows);
+    if (static_cast<long long>(cols) * 3 > 0x7FFFFFFFLL)
+        return fail(LLAMA2_ERR_UNSUPPORTED, "%s: cols=%d too large", fn, cols);
     return LLAMA2_OK;
 }
 
@@ -245,15 +325,39 @@ static int check_qweight(const char* fn, const char* name, const uint32_t* w, co
     return LLAMA2_OK;
 }
 
-template <bool RESIDUAL>
-static int launch_plain(const char* fn, int n_tensors, PlainArgs a, const llama2_half* input, int rows, int cols,
-                        int zs, int ss, int ws)
+template <int J, int MODE, int WAVES>
+static void launch_j(const Int4Args& a, int max_waves)
 {
-    constexpr int R = 2;
-    const dim3 grid(ceil_div(cols, kWaves * R), n_tensors);
-    const size_t lds = static_cast<size_t>(ws) * 16; // nchunks * 64 bytes
-    hipLaunchKernelGGL((int4_matvec_kernel<R, RESIDUAL>), grid, dim3(kThreads), lds, ctx().stream, a, input,
-                       rows, cols, ws, ss, zs);
+    const int nitems = a.n_tensors * a.N;
+    int waves = nitems < max_waves ? nitems : max_waves;
+    const int grid = ceil_div(waves, WAVES);
+    hipLaunchKernelGGL((int4_matvec_kernel<J, MODE, WAVES>), dim3(grid), dim3(WAVES * 64), 0, ctx().stream, a);
+}
+
+// Wavefronts kept resident per launch: 16 per CU while a lane holds up to 3
+// chunks of a row, 8 per CU for longer rows (more bytes in flight per lane).
+template <int MODE>
+static int launch_int4(const char* fn, const Int4Args& a)
+{
+    const int nchunks = a.ws / 4;
+    const int J = ceil_div(nchunks, 64);
+    const int cus = ctx().num_cus > 0 ? ctx().num_cus : 256;
+    switch (J) {
+    case 1: launch_j<1, MODE, 4>(a, cus * 16); break;
+    case 2: launch_j<2, MODE, 4>(a, cus * 16); break;
+    case 3: launch_j<3, MODE, 4>(a, cus * 16); break;
+    case 4: launch_j<4, MODE, 4>(a, cus * 8); break;
+    case 5: launch_j<5, MODE, 4>(a, cus * 8); break;
+    case 6: launch_j<6, MODE, 4>(a, cus * 8); break;
+    case 7: launch_j<7, MODE, 4>(a, cus * 8); break;
+    case 8: launch_j<8, MODE, 4>(a, cus * 8); break;
+    default: {
+        const int nitems = a.n_tensors * a.N;
+        const int grid = ceil_div(nitems < cus * 8 ? nitems : cus * 8, 4);
+        hipLaunchKernelGGL((int4_matvec_generic_kernel<MODE>), dim3(grid), dim3(256),
+                           static_cast<size_t>(nchunks) * 68, ctx().stream, a);
+    }
+    }
     L2_LAUNCH_CHECK(fn);
     return LLAMA2_OK;
 }
@@ -276,10 +380,12 @@ int llama2_mat_vec_residual_int4(llama2_half* output, const llama2_half* input, 
         return rc;
     L2_CHECK(!overlap(output, size_t(cols) * 2, input, size_t(rows) * 2),
              "%s: output overlaps input (other workgroups still read the input while rows are written)", fn);
-    PlainArgs a{};
+    Int4Args a{};
     a.m[0] = QW{weights, zeros, scales};
     a.out[0] = output;
-    return launch_plain<true>(fn, 1, a, input, rows, cols, zeros_size, scales_size, weights_size);
+    a.x = input;
+    a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 1;
+    return launch_int4<RESIDUAL>(fn, a);
 }
 
 int llama2_mat_vec_int4(llama2_half* output, const llama2_half* input, const uint32_t* weights,
@@ -293,10 +399,12 @@ int llama2_mat_vec_int4(llama2_half* output, const llama2_half* input, const uin
     if (int rc = check_qweight(fn, "matrix", weights, zeros, scales))
         return rc;
     L2_CHECK(!overlap(output, size_t(cols) * 2, input, size_t(rows) * 2), "%s: output overlaps input", fn);
-    PlainArgs a{};
+    Int4Args a{};
     a.m[0] = QW{weights, zeros, scales};
     a.out[0] = output;
-    return launch_plain<false>(fn, 1, a, input, rows, cols, zeros_size, scales_size, weights_size);
+    a.x = input;
+    a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 1;
+    return launch_int4<PLAIN>(fn, a);
 }
 
 int llama2_qkv_mat_vec(llama2_half* q_output, llama2_half* k_output, llama2_half* v_output,
@@ -319,14 +427,16 @@ int llama2_qkv_mat_vec(llama2_half* q_output, llama2_half* k_output, llama2_half
         return rc;
     for (llama2_half* o : {q_output, k_output, v_output})
         L2_CHECK(!overlap(o, size_t(cols) * 2, input, size_t(rows) * 2), "%s: an output overlaps the input", fn);
-    PlainArgs a{};
+    Int4Args a{};
     a.m[0] = QW{q_weight, q_zeros, q_scales};
     a.m[1] = QW{k_weight, k_zeros, k_scales};
     a.m[2] = QW{v_weight, v_zeros, v_scales};
     a.out[0] = q_output;
     a.out[1] = k_output;
     a.out[2] = v_output;
-    return launch_plain<false>(fn, 3, a, input, rows, cols, zeros_size, scales_size, weights_size);
+    a.x = input;
+    a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 3;
+    return launch_int4<PLAIN>(fn, a);
 }
 
 int llama2_mat_vec_swiglu(llama2_half* output, const llama2_half* input, const uint32_t* g_weight,
@@ -343,14 +453,13 @@ int llama2_mat_vec_swiglu(llama2_half* output, const llama2_half* input, const u
     if (int rc = check_qweight(fn, "up", u_weight, u_zeros, u_scales))
         return rc;
     L2_CHECK(!overlap(output, size_t(cols) * 2, input, size_t(rows) * 2), "%s: output overlaps input", fn);
-    constexpr int O = 1;
-    const dim3 grid(ceil_div(cols, kWaves * O));
-    const size_t lds = static_cast<size_t>(weights_size) * 16;
-    hipLaunchKernelGGL((int4_swiglu_kernel<O>), grid, dim3(kThreads), lds, ctx().stream,
-                       QW{g_weight, g_zeros, g_scales}, QW{u_weight, u_zeros, u_scales}, output, input, rows, cols,
-                       weights_size, scales_size, zeros_size);
-    L2_LAUNCH_CHECK(fn);
-    return LLAMA2_OK;
+    Int4Args a{};
+    a.m[0] = QW{g_weight, g_zeros, g_scales};
+    a.m[1] = QW{u_weight, u_zeros, u_scales};
+    a.out[0] = output;
+    a.x = input;
+    a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 1;
+    return launch_int4<SWIGLU>(fn, a);
 }
 
 } // extern "C"

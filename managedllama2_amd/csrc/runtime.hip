@@ -33,6 +33,9 @@ int ensure_attn_partials(size_t bytes)
     Context& c = ctx();
     if (bytes <= c.attn_partials_bytes)
         return LLAMA2_OK;
+    if (c.capturing)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT,
+                    "scratch of %zu bytes must exist before graph capture starts (run the call once eagerly first)", bytes);
     // Grow only between launches that use it: earlier kernels on the stream may
     // still read the old buffer, so drain the stream first.
     L2_HIP(hipStreamSynchronize(c.stream));
@@ -100,6 +103,8 @@ int llama2_shutdown(void)
 int llama2_malloc(void** ptr, size_t bytes)
 {
     L2_REQUIRE_INIT();
+    if (ctx().capturing)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_malloc: not allowed during graph capture");
     L2_CHECK(ptr != nullptr, "llama2_malloc: ptr is null");
     *ptr = nullptr;
     L2_CHECK(bytes > 0, "llama2_malloc: zero-sized allocation");
@@ -110,6 +115,8 @@ int llama2_malloc(void** ptr, size_t bytes)
 int llama2_free(void* ptr)
 {
     L2_REQUIRE_INIT();
+    if (ctx().capturing)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_free: not allowed during graph capture");
     if (!ptr)
         return LLAMA2_OK;
     L2_HIP(hipStreamSynchronize(ctx().stream));
@@ -120,6 +127,8 @@ int llama2_free(void* ptr)
 int llama2_memcpy_h2d(void* dst, size_t dst_offset_bytes, const void* src, size_t bytes)
 {
     L2_REQUIRE_INIT();
+    if (ctx().capturing)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_memcpy_h2d: not allowed during graph capture");
     if (bytes == 0)
         return LLAMA2_OK;
     L2_CHECK(dst && src, "llama2_memcpy_h2d: null pointer");
@@ -134,6 +143,8 @@ int llama2_memcpy_h2d(void* dst, size_t dst_offset_bytes, const void* src, size_
 int llama2_memcpy_d2h(void* dst, const void* src, size_t src_offset_bytes, size_t bytes)
 {
     L2_REQUIRE_INIT();
+    if (ctx().capturing)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_memcpy_d2h: not allowed during graph capture");
     if (bytes == 0)
         return LLAMA2_OK;
     L2_CHECK(dst && src, "llama2_memcpy_d2h: null pointer");
@@ -183,11 +194,66 @@ int llama2_mem_info(size_t* free_bytes, size_t* total_bytes)
 int llama2_sync(void)
 {
     L2_REQUIRE_INIT();
+    if (ctx().capturing)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_sync: not allowed during graph capture");
     L2_HIP(hipStreamSynchronize(ctx().stream));
     return LLAMA2_OK;
 }
 
 void* llama2_stream(void) { return ctx().ready ? static_cast<void*>(ctx().stream) : nullptr; }
+
+#define L2_NOT_CAPTURING(fn)                                                                  \
+    do {                                                                                      \
+        if (ctx().capturing)                                                                  \
+            return fail(LLAMA2_ERR_INVALID_ARGUMENT, fn ": not allowed during graph capture"); \
+    } while (0)
+
+int llama2_graph_begin_capture(void)
+{
+    L2_REQUIRE_INIT();
+    L2_NOT_CAPTURING("llama2_graph_begin_capture");
+    L2_HIP(hipStreamBeginCapture(ctx().stream, hipStreamCaptureModeThreadLocal));
+    ctx().capturing = true;
+    return LLAMA2_OK;
+}
+
+int llama2_graph_end_capture(void** graph)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(graph, "llama2_graph_end_capture: null pointer");
+    *graph = nullptr;
+    if (!ctx().capturing)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_graph_end_capture: no capture in progress");
+    ctx().capturing = false;
+    hipGraph_t g = nullptr;
+    L2_HIP(hipStreamEndCapture(ctx().stream, &g));
+    hipGraphExec_t exec = nullptr;
+    hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess)
+        return hip_fail(e, "hipGraphInstantiate");
+    *graph = exec;
+    return LLAMA2_OK;
+}
+
+int llama2_graph_launch(void* graph)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(graph, "llama2_graph_launch: null graph");
+    L2_NOT_CAPTURING("llama2_graph_launch");
+    L2_HIP(hipGraphLaunch(static_cast<hipGraphExec_t>(graph), ctx().stream));
+    return LLAMA2_OK;
+}
+
+int llama2_graph_destroy(void* graph)
+{
+    L2_REQUIRE_INIT();
+    if (!graph)
+        return LLAMA2_OK;
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    L2_HIP(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph)));
+    return LLAMA2_OK;
+}
 
 int llama2_event_create(void** event)
 {
