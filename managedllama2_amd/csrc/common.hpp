@@ -131,6 +131,69 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// Sum over a 256-thread workgroup (4 wavefronts), identical in every thread and
+// independent of which kernel calls it: RMSNorm is evaluated both by the
+// stand-alone module and inside the fused mat-vec kernels, and the two must
+// agree bit for bit.  `lds4` holds 4 floats.
+__device__ __forceinline__ float block256_sum(float v, float* lds4)
+{
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0)
+        lds4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    const float t = (lds4[0] + lds4[1]) + (lds4[2] + lds4[3]);
+    __syncthreads();
+    return t;
+}
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes)
+{
+    // raw buffer, 32-bit elements; out-of-range reads return 0
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, static_cast<int>(bytes), 0x00020000);
+}
+
+// One thread's share of a K-element fp16 vector read 16 bytes at a time by a
+// 256-thread workgroup: piece i covers elements 8*(tid + 256 i) .. +7.
+template <int PIECES>
+struct VecPieces {
+    u32x4 v[PIECES];
+    __device__ __forceinline__ void load(const uint16_t* p, int K)
+    {
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(p, K * 2);
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i)
+            v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, (threadIdx.x + i * 256) * 16, 0, 0);
+    }
+    __device__ __forceinline__ float sum_squares() const
+    {
+        float ss = 0.0f;
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const h2_t p = as_h2(v[i][k]);
+                const float a = static_cast<float>(p[0]), b = static_cast<float>(p[1]);
+                ss += a * a;
+                ss += b * b;
+            }
+        return ss;
+    }
+    // v <- half(rms * gamma * v), the product order of native/rmsnorm_kernel.cu:34
+    __device__ __forceinline__ void scale(float rms, const VecPieces& gamma)
+    {
+#pragma unroll
+        for (int i = 0; i < PIECES; ++i)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const h2_t x = as_h2(v[i][k]), g = as_h2(gamma.v[i][k]);
+                h2_t o;
+                o[0] = static_cast<_Float16>(rms * static_cast<float>(g[0]) * static_cast<float>(x[0]));
+                o[1] = static_cast<_Float16>(rms * static_cast<float>(g[1]) * static_cast<float>(x[1]));
+                v[i][k] = as_u32(o);
+            }
+    }
+};
+
 #endif // __HIPCC__
 
 } // namespace l2

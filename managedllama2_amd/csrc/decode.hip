@@ -1,11 +1,227 @@
 // The decode step: Transformer.Forward (src/Transformer.cs:158-190) with
 // MultiHeadAttention (:150-156) and the greedy branch of Sampler.Sample
 // (src/Sampler.cs:44-47,69), issued on the library's stream.
-#include "common.hpp"
+//
+// Two ways of issuing the step:
+//   LLAMA2_DECODE_MODULES  the reference's launch sequence, module by module
+//                          (1 + 10 L + 2 launches per token);
+//   LLAMA2_DECODE_FUSED    5 launches per layer: RMSNorm + QKV + RoPE + cache
+//                          write | split-sequence attention | o-proj + residual |
+//                          RMSNorm + SwiGLU | down-proj + residual.  Everything
+//                          that depends on the position is read from a small
+//                          device-resident state block, so the launch sequence
+//                          is identical for every token and can be replayed as
+//                          one hipGraph (LLAMA2_DECODE_GRAPH).
+#include "int4_kernels.hpp"
 
+#include <climits>
 #include <cmath>
 #include <new>
 #include <vector>
+
+namespace l2 {
+
+// ---------------------------------------------------------------- fused attention
+// One workgroup per (head, block of 128 timesteps).  Every byte of K and V the
+// workgroup needs is requested before the first score is computed (16 loads of
+// 16 bytes per lane), 16 lanes share one timestep, scores are rounded to fp16
+// like the reference's `attention` buffer, softmax statistics are per block and
+// the blocks of a head are merged by whichever workgroup finishes last
+// (fixed merge order: deterministic).
+constexpr int kSplitT = 128;
+constexpr int kPartStride = kRopeHeadSize + 2; // 128 partial outputs, block max, block sum
+
+struct AttnArgs {
+    const uint16_t* q;
+    const uint16_t* kcache; // layer base, rows of `dim` halfs
+    const uint16_t* vcache;
+    uint16_t* out; // [n_heads * 128]
+    float* part;   // [n_heads][max_splits][kPartStride]
+    unsigned* counters; // [n_heads], zero between launches
+    const int* pos_ptr;
+    int dim;
+    int max_splits;
+    float scale;
+};
+
+__global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
+{
+    __shared__ float sc[kSplitT];
+    __shared__ float red[16][kRopeHeadSize];
+    __shared__ int is_last;
+    const int split = blockIdx.x, h = blockIdx.y;
+    const int S = a.pos_ptr[0] + 1; // attends rows 0..pos (src/Transformer.cs:175)
+    const int nsplit = (S + kSplitT - 1) / kSplitT;
+    if (split >= nsplit)
+        return;
+    const int t0 = split * kSplitT;
+    const int t1 = S < t0 + kSplitT ? S : t0 + kSplitT;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l16 = lane & 15, grp = wave * 4 + (lane >> 4);
+    const size_t col = static_cast<size_t>(h) * kRopeHeadSize + l16 * 8;
+
+    const u32x4 qv = *reinterpret_cast<const u32x4*>(a.q + col);
+    u32x4 kv[8], vv[8];
+    bool ok[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int t = t0 + i * 16 + grp;
+        ok[i] = t < t1;
+        const size_t off = static_cast<size_t>(ok[i] ? t : t0) * a.dim + col;
+        kv[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.kcache + off));
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int t = t0 + i * 16 + grp;
+        const size_t off = static_cast<size_t>(ok[i] ? t : t0) * a.dim + col;
+        vv[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.vcache + off));
+    }
+    float s[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            acc = dot2(kv[i][k], qv[k], acc);
+        acc = row16_sum(acc) * a.scale; // native/mat_vec_kernel.cu:71-74
+        s[i] = ok[i] ? half_bits_to_float(float_to_half_bits(acc)) : -INFINITY;
+        if (l16 == 0)
+            sc[i * 16 + grp] = s[i];
+    }
+    __syncthreads();
+    const float m = wave_max(fmaxf(sc[lane], sc[lane + 64]));
+    const float l = wave_sum(expf(sc[lane] - m) + expf(sc[lane + 64] - m));
+    float o[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        o[k] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float p = expf(s[i] - m); // 0 for masked timesteps
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const h2_t v2 = as_h2(vv[i][k]);
+            o[2 * k] = fmaf(p, static_cast<float>(v2[0]), o[2 * k]);
+            o[2 * k + 1] = fmaf(p, static_cast<float>(v2[1]), o[2 * k + 1]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        red[grp][l16 * 8 + k] = o[k];
+    __syncthreads();
+    float val = 0.0f;
+    if (threadIdx.x < kRopeHeadSize) {
+#pragma unroll
+        for (int g = 0; g < 16; ++g)
+            val += red[g][threadIdx.x];
+    }
+    uint16_t* out = a.out + static_cast<size_t>(h) * kRopeHeadSize;
+    if (nsplit == 1) {
+        if (threadIdx.x < kRopeHeadSize)
+            out[threadIdx.x] = float_to_half_bits(val / l);
+        return;
+    }
+    float* P = a.part + (static_cast<size_t>(h) * a.max_splits + split) * kPartStride;
+    if (threadIdx.x < kRopeHeadSize)
+        P[threadIdx.x] = val;
+    if (threadIdx.x == 0) {
+        P[kRopeHeadSize] = m;
+        P[kRopeHeadSize + 1] = l;
+    }
+    __threadfence(); // publish the partials before announcing them
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned prev = atomicAdd(&a.counters[h], 1u);
+        is_last = prev == static_cast<unsigned>(nsplit - 1);
+    }
+    __syncthreads();
+    if (!is_last)
+        return;
+    __threadfence(); // see every other block's partials
+    if (threadIdx.x == 0)
+        a.counters[h] = 0; // ready for the next launch
+    if (threadIdx.x < kRopeHeadSize) {
+        const float* P0 = a.part + static_cast<size_t>(h) * a.max_splits * kPartStride;
+        float M = -INFINITY;
+        for (int i = 0; i < nsplit; ++i)
+            M = fmaxf(M, P0[i * kPartStride + kRopeHeadSize]);
+        float L = 0.0f, O = 0.0f;
+        for (int i = 0; i < nsplit; ++i) {
+            const float w = expf(P0[i * kPartStride + kRopeHeadSize] - M);
+            L = fmaf(w, P0[i * kPartStride + kRopeHeadSize + 1], L);
+            O = fmaf(w, P0[i * kPartStride + threadIdx.x], O);
+        }
+        out[threadIdx.x] = float_to_half_bits(O / L);
+    }
+}
+
+// ---------------------------------------------------------------- step state
+// state[0] = position, state[1] = first position whose token is generated,
+// state[2] = 1 to advance the position after sampling.
+__global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance)
+{
+    state[0] = pos;
+    state[1] = n_prompt;
+    state[2] = advance;
+}
+
+__device__ __forceinline__ bool better(float va, int ia, float vb, int ib)
+{
+    return va > vb || (va == vb && ia < ib);
+}
+
+// Sampler.Sample greedy branch (src/Sampler.cs:44-47) against the device state:
+// tokens[pos+1] = argmax(logits) iff pos+1 >= n_prompt; lowest index wins ties.
+__global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, int size, int* tokens, int* state)
+{
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    float bv = -INFINITY;
+    int bi = INT_MAX;
+    for (int i = threadIdx.x; i < size; i += 1024) {
+        const float f = half_bits_to_float(x[i]);
+        if (better(f, i, bv, bi)) {
+            bv = f;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (better(ov, oi, bv, bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        sv[threadIdx.x >> 6] = bv;
+        si[threadIdx.x >> 6] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        bv = threadIdx.x < 16 ? sv[threadIdx.x] : -INFINITY;
+        bi = threadIdx.x < 16 ? si[threadIdx.x] : INT_MAX;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (better(ov, oi, bv, bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+        if (threadIdx.x == 0) {
+            const int pos = state[0];
+            if (pos + 1 >= state[1])
+                tokens[pos + 1] = bi == INT_MAX ? 0 : bi;
+            if (state[2])
+                state[0] = pos + 1;
+        }
+    }
+}
+
+} // namespace l2
 
 struct llama2_decoder {
     llama2_config cfg;
@@ -15,6 +231,13 @@ struct llama2_decoder {
     int mode;
     int kv_dim;
     int head_size;
+    // fused path
+    int* state = nullptr;
+    float* attn_part = nullptr;
+    unsigned* counters = nullptr;
+    int max_splits = 0;
+    hipGraphExec_t graph_forward = nullptr; // Transformer.Forward
+    hipGraphExec_t graph_step = nullptr;    // Forward + greedy sample + position advance
 };
 
 using namespace l2;
@@ -25,6 +248,7 @@ int check_qw(const llama2_qweight& q, const char* what, int layer)
 {
     L2_CHECK(q.weight && q.zeros && q.scales, "llama2_decode_create: layer %d %s tensor has a null pointer", layer,
              what);
+    L2_CHECK(aligned(q.weight, 16), "llama2_decode_create: layer %d %s weights must be 16-byte aligned", layer, what);
     return LLAMA2_OK;
 }
 
@@ -75,6 +299,120 @@ int forward_modules(llama2_decoder* d, int position, int next_position)
     return LLAMA2_OK;
 }
 
+QW qw(const llama2_qweight& q) { return QW{q.weight, q.zeros, q.scales}; }
+
+// The same step in 5 launches per layer; the position comes from d->state.
+int forward_fused(llama2_decoder* d)
+{
+    const llama2_config& c = d->cfg;
+    const llama2_run_state& s = d->s;
+    const int dim = c.dim, hidden = c.hidden_dim;
+    const int ss = ceil_div(dim, 128), ws = ceil_div(dim, 32) * 4, zs = ceil_div(ss, 8);
+    const int hss = ceil_div(hidden, 128), hws = ceil_div(hidden, 32) * 4, hzs = ceil_div(hss, 8);
+    for (int i = 0; i < c.n_layers; ++i) {
+        const llama2_layer_weights& L = d->layers[i];
+        const size_t layer_offset = static_cast<size_t>(i) * c.seq_len * d->kv_dim;
+        {
+            Int4Args a{}; // :163 (layer 0) + :167 + :171 + :173
+            a.m[0] = qw(L.query), a.m[1] = qw(L.key), a.m[2] = qw(L.value);
+            a.out[0] = s.q, a.out[1] = s.key_cache + layer_offset, a.out[2] = s.value_cache + layer_offset;
+            a.x = s.x;
+            a.K = dim, a.N = dim, a.ws = ws, a.ss = ss, a.zs = zs, a.n_tensors = 3;
+            a.gamma = L.rms_attention, a.eps = 1e-5f;
+            if (i == 0)
+                a.embedding = d->w.token_embedding_table, a.tokens = s.tokens, a.vocab = c.vocab_size, a.x_out = s.x;
+            a.pos_ptr = d->state;
+            a.kv_dim = d->kv_dim, a.theta = c.rope_theta;
+            L2_TRY((launch_int4<QKV_ROPE, STAGE_RMSNORM>("fused qkv", a)));
+        }
+        {
+            AttnArgs a{}; // :175 (MultiHeadAttention :150-156)
+            a.q = s.q, a.kcache = s.key_cache + layer_offset, a.vcache = s.value_cache + layer_offset, a.out = s.xb;
+            a.part = d->attn_part, a.counters = d->counters, a.pos_ptr = d->state;
+            a.dim = dim, a.max_splits = d->max_splits;
+            a.scale = 1.0f / sqrtf(static_cast<float>(d->head_size));
+            hipLaunchKernelGGL(fused_attn_kernel, dim3(d->max_splits, c.n_heads), dim3(256), 0, ctx().stream, a);
+            L2_LAUNCH_CHECK("fused attention");
+        }
+        {
+            Int4Args a{}; // :177
+            a.m[0] = qw(L.output), a.out[0] = s.x, a.x = s.xb;
+            a.K = dim, a.N = dim, a.ws = ws, a.ss = ss, a.zs = zs, a.n_tensors = 1;
+            L2_TRY((launch_int4<RESIDUAL, STAGE_X>("fused o-proj", a)));
+        }
+        {
+            Int4Args a{}; // :179 + :181
+            a.m[0] = qw(L.gate), a.m[1] = qw(L.up), a.out[0] = s.h, a.x = s.x;
+            a.K = dim, a.N = hidden, a.ws = ws, a.ss = ss, a.zs = zs, a.n_tensors = 1;
+            a.gamma = L.rms_feed_forward, a.eps = 1e-5f;
+            L2_TRY((launch_int4<SWIGLU, STAGE_RMSNORM>("fused swiglu", a)));
+        }
+        {
+            Int4Args a{}; // :183
+            a.m[0] = qw(L.down), a.out[0] = s.x, a.x = s.h;
+            a.K = hidden, a.N = dim, a.ws = hws, a.ss = hss, a.zs = hzs, a.n_tensors = 1;
+            L2_TRY((launch_int4<RESIDUAL, STAGE_X>("fused down-proj", a)));
+        }
+    }
+    L2_TRY(llama2_rmsnorm(s.x, s.x, d->w.rms_final_weight, dim, 1e-5f)); // :187
+    L2_TRY(llama2_mat_vec(s.logits, s.x, d->w.classifier_weights, dim, c.vocab_size)); // :189
+    return LLAMA2_OK;
+}
+
+int launch_argmax_step(llama2_decoder* d)
+{
+    hipLaunchKernelGGL(argmax_step_kernel, dim3(1), dim3(1024), 0, ctx().stream, d->s.logits, d->cfg.vocab_size,
+                       d->s.tokens, d->state);
+    L2_LAUNCH_CHECK("argmax_step_kernel");
+    return LLAMA2_OK;
+}
+
+int set_state(llama2_decoder* d, int pos, int n_prompt, int advance)
+{
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx().stream, d->state, pos, n_prompt, advance);
+    L2_LAUNCH_CHECK("set_state_kernel");
+    return LLAMA2_OK;
+}
+
+int capture(hipGraphExec_t* exec, llama2_decoder* d, bool with_sample)
+{
+    L2_HIP(hipStreamBeginCapture(ctx().stream, hipStreamCaptureModeThreadLocal));
+    ctx().capturing = true;
+    int rc = forward_fused(d);
+    if (rc == LLAMA2_OK && with_sample)
+        rc = launch_argmax_step(d);
+    ctx().capturing = false;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx().stream, &g);
+    if (rc != LLAMA2_OK) {
+        if (g)
+            (void)hipGraphDestroy(g);
+        return rc;
+    }
+    if (e != hipSuccess)
+        return hip_fail(e, "hipStreamEndCapture");
+    e = hipGraphInstantiate(exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess)
+        return hip_fail(e, "hipGraphInstantiate");
+    return LLAMA2_OK;
+}
+
+void release(llama2_decoder* d)
+{
+    if (d->graph_forward)
+        (void)hipGraphExecDestroy(d->graph_forward);
+    if (d->graph_step)
+        (void)hipGraphExecDestroy(d->graph_step);
+    if (d->state)
+        (void)hipFree(d->state);
+    if (d->attn_part)
+        (void)hipFree(d->attn_part);
+    if (d->counters)
+        (void)hipFree(d->counters);
+    delete d;
+}
+
 } // namespace
 
 extern "C" {
@@ -86,6 +424,7 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     const char* fn = "llama2_decode_create";
     L2_CHECK(decoder && config && weights && state, "%s: null argument", fn);
     *decoder = nullptr;
+    L2_CHECK(!ctx().capturing, "%s: not allowed during graph capture", fn);
     const llama2_config& c = *config;
     L2_CHECK(c.dim > 0 && c.hidden_dim > 0 && c.n_layers > 0 && c.n_heads > 0 && c.n_kv_heads > 0 &&
                  c.vocab_size > 0 && c.seq_len > 0,
@@ -100,7 +439,21 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     if (c.seq_len > LLAMA2_MAX_SOFTMAX_SIZE)
         return fail(LLAMA2_ERR_UNSUPPORTED, "%s: seq_len=%d exceeds the softmax limit %d", fn, c.seq_len,
                     LLAMA2_MAX_SOFTMAX_SIZE);
-    L2_CHECK(mode == LLAMA2_DECODE_MODULES, "%s: unknown mode %d", fn, mode);
+    L2_CHECK(mode >= 0 && mode <= (LLAMA2_DECODE_FUSED | LLAMA2_DECODE_GRAPH), "%s: unknown mode %d", fn, mode);
+    const bool fused = (mode & LLAMA2_DECODE_FUSED) != 0;
+    if ((mode & LLAMA2_DECODE_GRAPH) && !fused)
+        return fail(LLAMA2_ERR_UNSUPPORTED,
+                    "%s: LLAMA2_DECODE_GRAPH needs LLAMA2_DECODE_FUSED (the module sequence takes the position by value)", fn);
+    if (fused) {
+        const int head_size = c.dim / c.n_heads;
+        if (head_size != kRopeHeadSize || c.dim % 8 || c.hidden_dim % 8 ||
+            chunk_columns(ceil_div(c.dim, 32) * 4) > kMaxChunkColumns ||
+            chunk_columns(ceil_div(c.hidden_dim, 32) * 4) > kMaxChunkColumns)
+            return fail(LLAMA2_ERR_UNSUPPORTED,
+                        "%s: the fused step needs head_size 128 and dim, hidden_dim multiples of 8 up to 16384 "
+                        "(got head_size %d, dim %d, hidden_dim %d); use LLAMA2_DECODE_MODULES",
+                        fn, head_size, c.dim, c.hidden_dim);
+    }
     L2_CHECK(weights->token_embedding_table && weights->classifier_weights && weights->rms_final_weight &&
                  weights->layers,
              "%s: null pointer in weights", fn);
@@ -118,6 +471,10 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     L2_CHECK(state->x && state->xb && state->h && state->q && state->attention && state->logits &&
                  state->key_cache && state->value_cache && state->tokens,
              "%s: null pointer in run state", fn);
+    for (const void* p : {static_cast<const void*>(state->x), static_cast<const void*>(state->xb),
+                          static_cast<const void*>(state->h), static_cast<const void*>(state->q),
+                          static_cast<const void*>(state->key_cache), static_cast<const void*>(state->value_cache)})
+        L2_CHECK(aligned(p, 16), "%s: run-state buffers must be 16-byte aligned", fn);
     llama2_decoder* d = new (std::nothrow) llama2_decoder();
     L2_CHECK(d, "%s: out of host memory", fn);
     d->cfg = c;
@@ -128,6 +485,34 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     d->mode = mode;
     d->kv_dim = kv_dim;
     d->head_size = c.dim / c.n_heads;
+    if (fused) {
+        d->max_splits = ceil_div(c.seq_len, kSplitT);
+        hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->state), 4 * sizeof(int));
+        if (e == hipSuccess)
+            e = hipMalloc(reinterpret_cast<void**>(&d->attn_part),
+                          sizeof(float) * static_cast<size_t>(c.n_heads) * d->max_splits * kPartStride);
+        if (e == hipSuccess)
+            e = hipMalloc(reinterpret_cast<void**>(&d->counters), sizeof(unsigned) * c.n_heads);
+        if (e == hipSuccess)
+            e = hipMemsetAsync(d->counters, 0, sizeof(unsigned) * c.n_heads, ctx().stream);
+        if (e == hipSuccess)
+            e = hipMemsetAsync(d->state, 0, 4 * sizeof(int), ctx().stream);
+        if (e == hipSuccess)
+            e = hipStreamSynchronize(ctx().stream);
+        if (e != hipSuccess) {
+            release(d);
+            return hip_fail(e, "llama2_decode_create: scratch allocation");
+        }
+        if (mode & LLAMA2_DECODE_GRAPH) {
+            int rc = capture(&d->graph_forward, d, false);
+            if (rc == LLAMA2_OK)
+                rc = capture(&d->graph_step, d, true);
+            if (rc != LLAMA2_OK) {
+                release(d);
+                return rc;
+            }
+        }
+    }
     *decoder = d;
     return LLAMA2_OK;
 }
@@ -140,7 +525,14 @@ int llama2_decode_forward(llama2_decoder* d, int position, int next_position)
              position, d->cfg.seq_len);
     L2_CHECK(next_position == position + 1, "llama2_decode_forward: next_position=%d must be position+1=%d",
              next_position, position + 1);
-    return forward_modules(d, position, next_position);
+    if (!(d->mode & LLAMA2_DECODE_FUSED))
+        return forward_modules(d, position, next_position);
+    L2_TRY(set_state(d, position, INT_MAX, 0));
+    if (d->graph_forward) {
+        L2_HIP(hipGraphLaunch(d->graph_forward, ctx().stream));
+        return LLAMA2_OK;
+    }
+    return forward_fused(d);
 }
 
 int llama2_decode_sample(llama2_decoder* d, int next_position, int generate_token, int* token)
@@ -159,9 +551,21 @@ int llama2_decode_run(llama2_decoder* d, int position, int steps, int n_prompt)
     L2_CHECK(d, "llama2_decode_run: null decoder");
     L2_CHECK(position >= 0 && steps >= 0 && position + steps <= d->cfg.seq_len,
              "llama2_decode_run: position=%d steps=%d exceed seq_len=%d", position, steps, d->cfg.seq_len);
-    for (int pos = position; pos < position + steps; ++pos) {
-        L2_TRY(forward_modules(d, pos, pos + 1));
-        L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, d->s.tokens, pos + 1, pos + 1 >= n_prompt));
+    if (!(d->mode & LLAMA2_DECODE_FUSED)) {
+        for (int pos = position; pos < position + steps; ++pos) {
+            L2_TRY(forward_modules(d, pos, pos + 1));
+            L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, d->s.tokens, pos + 1, pos + 1 >= n_prompt));
+        }
+        return LLAMA2_OK;
+    }
+    L2_TRY(set_state(d, position, n_prompt, 1));
+    for (int i = 0; i < steps; ++i) {
+        if (d->graph_step) {
+            L2_HIP(hipGraphLaunch(d->graph_step, ctx().stream));
+        } else {
+            L2_TRY(forward_fused(d));
+            L2_TRY(launch_argmax_step(d));
+        }
     }
     return LLAMA2_OK;
 }
@@ -172,7 +576,7 @@ int llama2_decode_destroy(llama2_decoder* d)
         return LLAMA2_OK;
     if (ctx().ready)
         L2_HIP(hipStreamSynchronize(ctx().stream));
-    delete d;
+    release(d);
     return LLAMA2_OK;
 }
 

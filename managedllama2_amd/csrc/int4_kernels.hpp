@@ -1,0 +1,417 @@
+// AWQ-v1 int4 (group 128) mat-vec kernels for gfx950, shared by the module entry
+// points (int4_matvec.hip) and the fused decode step (decode.hip).
+// Replaces native/mat_vec_kernel.cu:83-234 of the reference.
+//
+// Shape of the computation (batch-1 GEMV, HBM-bound, no MFMA):
+//   * a "chunk" is 16 bytes of one weight row = 4 uint32 = 32 nibbles; a
+//     64-lane wavefront reads 64 consecutive chunks (1 KiB) per load
+//     instruction, lane l taking chunks l, l+64, ... (buffer_load_dwordx4
+//     through a per-row buffer resource, so the ragged end of a row reads as
+//     zero without any lane predication);
+//   * wavefronts are persistent: each walks over its rows with the next row's
+//     loads already in flight while the current one is reduced;
+//   * the input vector is staged once per workgroup in LDS, pre-permuted to
+//     the order the nibble extraction produces, in four planes so that
+//     consecutive lanes read consecutive 16-byte slots (conflict-free
+//     ds_read_b128), together with the fp32 sum of every 32-element chunk.
+//     The staging step can apply RMSNorm on the way (fused decode step);
+//   * a nibble masked in place (w & 0x000F000F, w & 0x00F000F0) IS an fp16
+//     subnormal pair (n * 2^-24 resp. n * 2^-20): v_dot2_f32_f16 multiplies it
+//     exactly with the fp16 input pair and accumulates in fp32, so dequantising
+//     costs one v_and per pair.  The zero-point is applied per chunk as
+//     -z * sum(x), the group scale once per chunk, all in fp32;
+//   * lanes are reduced with DPP row operations.
+#pragma once
+
+#include "common.hpp"
+
+namespace l2 {
+
+struct QW {
+    const uint32_t* w;
+    const uint32_t* z;
+    const uint16_t* s;
+};
+
+// What the wavefront does with its dot products.
+enum Mode {
+    PLAIN = 0,    // out[t][n] = half(sum)                     (1 or 3 tensors)
+    RESIDUAL = 1, // out[0][n] = half(sum + float(out[0][n]))
+    SWIGLU = 2,   // out[0][n] = half(silu(gate.x) * (up.x))
+    QKV_ROPE = 3, // q/k/v rows (i, i+64) of a head; q and k rotated; k, v written to the cache row of *pos
+};
+// Where the staged input comes from.
+enum Stage {
+    STAGE_X = 0,       // x as given
+    STAGE_RMSNORM = 1, // half(rms * gamma * x), x = a.x or (layer 0) the embedding row of tokens[*pos]
+};
+
+constexpr int kRopeHeadSize = 128; // QKV_ROPE assumes head_size 128 (pairs i, i+64)
+
+struct Int4Args {
+    QW m[3];          // PLAIN/RESIDUAL: m[0] (QKV: q,k,v); SWIGLU: gate, up
+    uint16_t* out[3]; // one output vector per tensor; QKV_ROPE: q, key-cache layer base, value-cache layer base
+    const uint16_t* x;
+    int K, N, ws, ss, zs;
+    int n_tensors;
+    // STAGE_RMSNORM
+    const uint16_t* gamma;
+    float eps;
+    const uint16_t* embedding; // non-null: x = embedding[tokens[*pos] * K ..], also copied to x_out
+    const int* tokens;
+    int vocab;
+    uint16_t* x_out;
+    // device-resident step state: pos_ptr[0] = position
+    const int* pos_ptr;
+    // QKV_ROPE
+    int kv_dim;
+    float theta;
+};
+
+constexpr int kAuxStream = 2; // "nt": weights are touched once
+
+template <int J, int R>
+struct Frag { // what one lane holds of R rows: J chunks each + its group's zero word and scale
+    u32x4 w[R][J];
+    uint32_t zw[R][J];
+    uint16_t sb[R][J];
+};
+
+template <int J>
+__device__ __forceinline__ void load_row(u32x4 (&w)[J], uint32_t (&zw)[J], uint16_t (&sb)[J], const QW& m,
+                                         size_t row, int ws, int ss, int zs, int lane)
+{
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(m.w + row * ws, ws * 4);
+    const __amdgpu_buffer_rsrc_t rz = make_rsrc(m.z + row * zs, zs * 4);
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.s + row * ss, ss * 2);
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        // chunk c = lane + 64 j: group c/4, zero word c/32
+        w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
+        zw[j] = __builtin_amdgcn_raw_buffer_load_b32(rz, (lane >> 5) * 4 + j * 8, 0, 0);
+        sb[j] = __builtin_amdgcn_raw_buffer_load_b16(rs, (lane >> 2) * 2 + j * 32, 0, 0);
+    }
+}
+
+// LDS image of the input for J chunk-columns per lane:
+//   xs[i*JC + c] holds elements 8*(4c+i)+{0,4,1,5,2,6,3,7} (JC = 64 J, zero beyond K),
+//   sx[c] the fp32 sum of the 32 elements of chunk c.
+template <int J>
+__device__ __forceinline__ void commit_pieces(u32x4* xs, float* sx, const VecPieces<J>& p)
+{
+    constexpr int JC = J * 64;
+#pragma unroll
+    for (int i = 0; i < J; ++i) { // JC*4 pieces over 256 threads = J per thread
+        const int e = threadIdx.x + i * 256;
+        const u32x4 v = p.v[i];
+        u32x4 o;
+        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);     // x0,x4
+        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u); // x1,x5
+        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);     // x2,x6
+        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u); // x3,x7
+        xs[(e & 3) * JC + (e >> 2)] = o;
+        const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
+        s += dpp_f32<DPP_QUAD_XOR1>(s); // the 4 words of a chunk sit in one quad of lanes
+        s += dpp_f32<DPP_QUAD_XOR2>(s);
+        if ((e & 3) == 0)
+            sx[e >> 2] = s;
+    }
+}
+
+// Dot products of R rows (J chunks per lane each) with the staged input.
+template <int J, int R>
+__device__ __forceinline__ void dot_frag(float (&acc)[R], const Frag<J, R>& f, const u32x4* xs, const float* sx,
+                                         int lane, int zshift)
+{
+    constexpr int JC = J * 64;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+        acc[r] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        const int c = lane + 64 * j;
+        u32x4 xv[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            xv[i] = xs[i * JC + c];
+        const float sxv = sx[c];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float a0 = 0.0f, a1 = 0.0f; // a0: nibbles at bit 0 of a byte (x 2^-24), a1: at bit 4 (x 2^-20)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t w = f.w[r][j][i], w8 = w >> 8;
+                a0 = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[i][0]), a0, false);  // n0,n4
+                a1 = __builtin_amdgcn_fdot2(as_h2(w & 0x00F000F0u), as_h2(xv[i][1]), a1, false);  // n1,n5
+                a0 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[i][2]), a0, false); // n2,n6
+                a1 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), as_h2(xv[i][3]), a1, false); // n3,n7
+            }
+            const float zf = static_cast<float>((f.zw[r][j] >> zshift) & 0xFu);
+            float t = a0 * 16777216.0f;  // 2^24
+            t = fmaf(a1, 1048576.0f, t); // 2^20
+            t = fmaf(-zf, sxv, t);       // sum x (n - z)
+            acc[r] = fmaf(t, half_bits_to_float(f.sb[r][j]), acc[r]);
+        }
+    }
+}
+
+// cos/sin of pos * theta^(-2i/head_size) for i < head_size/2, the float
+// expression of native/rope_kernel.cu:8-12.
+__device__ __forceinline__ void rope_cos_sin(float& fcr, float& fci, int i, int head_size, int pos, float theta)
+{
+    const int head_dim = (i * 2) % head_size;
+    const float freq = 1.0f / powf(theta, static_cast<float>(head_dim) / static_cast<float>(head_size));
+    const float val = static_cast<float>(pos) * freq;
+    fcr = cosf(val);
+    fci = sinf(val);
+}
+
+template <int J, int MODE, int STAGE>
+__global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
+{
+    constexpr int R = (MODE == SWIGLU || MODE == QKV_ROPE) ? 2 : 1;
+    constexpr int JC = J * 64;
+    constexpr int WAVES = 4;
+    __shared__ u32x4 xs[4 * JC];
+    __shared__ float sx[JC];
+    __shared__ float red4[4];
+    __shared__ float rope_tab[MODE == QKV_ROPE ? kRopeHeadSize : 2]; // (cos, sin) pairs
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int total_waves = gridDim.x * WAVES;
+    const int pos = (MODE == QKV_ROPE || STAGE == STAGE_RMSNORM) && a.pos_ptr ? a.pos_ptr[0] : 0;
+    const int pairs = a.N >> 1; // QKV_ROPE: (i, i+64) row pairs per tensor
+    const int nitems = MODE == QKV_ROPE ? 3 * pairs : a.n_tensors * a.N;
+    int item = blockIdx.x * WAVES + wave;
+
+    auto load_item = [&](Frag<J, R>& f, uint16_t& res, int it) {
+        it = __builtin_amdgcn_readfirstlane(it);
+        if (MODE == SWIGLU) {
+            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[0], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
+            load_row<J>(f.w[R - 1], f.zw[R - 1], f.sb[R - 1], a.m[1], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
+        } else if (MODE == QKV_ROPE) {
+            const int t = (it >= pairs) + (it >= 2 * pairs), rem = it - t * pairs;
+            const int n0 = (rem >> 6) * kRopeHeadSize + (rem & 63);
+            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[t], static_cast<size_t>(n0), a.ws, a.ss, a.zs, lane);
+            load_row<J>(f.w[R - 1], f.zw[R - 1], f.sb[R - 1], a.m[t], static_cast<size_t>(n0 + 64), a.ws, a.ss, a.zs,
+                        lane);
+        } else {
+            const int t = (it >= a.N) + (it >= 2 * a.N), n = it - t * a.N; // at most 3 tensors
+            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[t], static_cast<size_t>(n), a.ws, a.ss, a.zs, lane);
+            if (MODE == RESIDUAL)
+                res = a.out[t][n];
+        }
+    };
+
+    // input first (served by L2), then the first item's weights (HBM)
+    VecPieces<J> xp;
+    const uint16_t* xsrc = a.x;
+    if (STAGE == STAGE_RMSNORM && a.embedding) { // native/embedding_kernel.cu:9-11
+        int token = a.tokens[pos];
+        token = token < 0 ? 0 : (token >= a.vocab ? a.vocab - 1 : token); // never read outside the table
+        xsrc = a.embedding + static_cast<size_t>(token) * a.K;
+    }
+    xp.load(xsrc, a.K);
+    VecPieces<J> gp;
+    if (STAGE == STAGE_RMSNORM)
+        gp.load(a.gamma, a.K);
+    Frag<J, R> cur;
+    uint16_t cur_res = 0;
+    if (item < nitems)
+        load_item(cur, cur_res, item);
+
+    if (MODE == QKV_ROPE && threadIdx.x < kRopeHeadSize / 2) {
+        float c, s;
+        rope_cos_sin(c, s, threadIdx.x, kRopeHeadSize, pos, a.theta);
+        rope_tab[2 * threadIdx.x] = c;
+        rope_tab[2 * threadIdx.x + 1] = s;
+    }
+    if (STAGE == STAGE_RMSNORM) {
+        if (a.embedding && blockIdx.x == 0) { // the residual stream starts as the embedding row
+            const __amdgpu_buffer_rsrc_t ro = make_rsrc(a.x_out, a.K * 2);
+#pragma unroll
+            for (int i = 0; i < J; ++i)
+                __builtin_amdgcn_raw_buffer_store_b128(xp.v[i], ro, (threadIdx.x + i * 256) * 16, 0, 0);
+        }
+        const float ss = block256_sum(xp.sum_squares(), red4);
+        const float rms = 1.0f / sqrtf(ss / static_cast<float>(a.K) + a.eps); // native/rmsnorm_kernel.cu:25-27
+        xp.scale(rms, gp);
+    }
+    commit_pieces<J>(xs, sx, xp);
+    __syncthreads();
+
+    const int zshift = ((lane >> 2) & 7) * 4; // nibble of the zero word: group (c/4) % 8, same for every j
+    for (; item < nitems; item += total_waves) {
+        Frag<J, R> nxt;
+        uint16_t nxt_res = 0;
+        if (item + total_waves < nitems)
+            load_item(nxt, nxt_res, item + total_waves);
+        float acc[R];
+        dot_frag<J, R>(acc, cur, xs, sx, lane, zshift);
+        if (MODE == SWIGLU) {
+            const float g = wave_sum(acc[0]);
+            const float u = wave_sum(acc[R - 1]);
+            if (lane == 0) {
+                float v = g;
+                v *= 1.0f / (1.0f + expf(-v)); // native/mat_vec_kernel.cu:219-221
+                v *= u;
+                a.out[0][item] = float_to_half_bits(v);
+            }
+        } else if (MODE == QKV_ROPE) {
+            // the unfused path stores q/k as fp16 and RoPE reads them back: keep that rounding
+            const float v0 = half_bits_to_float(float_to_half_bits(wave_sum(acc[0])));
+            const float v1 = half_bits_to_float(float_to_half_bits(wave_sum(acc[R - 1])));
+            if (lane == 0) {
+                const int t = (item >= pairs) + (item >= 2 * pairs), rem = item - t * pairs;
+                const int i = rem & 63, n0 = (rem >> 6) * kRopeHeadSize + i;
+                uint16_t* dst = t == 0 ? a.out[0] : a.out[t] + static_cast<size_t>(pos) * a.kv_dim;
+                float o0 = v0, o1 = v1;
+                if (t < 2) { // native/rope_kernel.cu:14-26
+                    const float fcr = rope_tab[2 * i], fci = rope_tab[2 * i + 1];
+                    o0 = v0 * fcr - v1 * fci;
+                    o1 = v0 * fci + v1 * fcr;
+                }
+                dst[n0] = float_to_half_bits(o0);
+                dst[n0 + 64] = float_to_half_bits(o1);
+            }
+        } else {
+            float v = wave_sum(acc[0]);
+            if (lane == 0) {
+                const int t = (item >= a.N) + (item >= 2 * a.N), n = item - t * a.N;
+                if (MODE == RESIDUAL)
+                    v += half_bits_to_float(cur_res);
+                a.out[t][n] = float_to_half_bits(v);
+            }
+        }
+        cur = nxt;
+        cur_res = nxt_res;
+    }
+}
+
+// Any K (fallback beyond 8 chunk-columns per lane): runtime trip count, dynamic LDS.
+template <int MODE>
+__global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
+{
+    constexpr int R = MODE == SWIGLU ? 2 : 1;
+    extern __shared__ u32x4 xs_dyn[];
+    const int nchunks = a.ws >> 2;
+    float* sx = reinterpret_cast<float*>(xs_dyn + 4 * nchunks);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int total_waves = gridDim.x * 4;
+    const int nitems = a.n_tensors * a.N;
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, a.K * 2);
+    for (int e = threadIdx.x; e < nchunks * 4; e += 256) {
+        const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rx, e * 16, 0, 0);
+        u32x4 o;
+        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);
+        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u);
+        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);
+        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u);
+        xs_dyn[(e & 3) * nchunks + (e >> 2)] = o;
+        const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
+        s += dpp_f32<DPP_QUAD_XOR1>(s);
+        s += dpp_f32<DPP_QUAD_XOR2>(s);
+        if ((e & 3) == 0)
+            sx[e >> 2] = s;
+    }
+    __syncthreads();
+    const int zshift = ((lane >> 2) & 7) * 4;
+    for (int item = blockIdx.x * 4 + wave; item < nitems; item += total_waves) {
+        const int it = __builtin_amdgcn_readfirstlane(item);
+        const int t = MODE == SWIGLU ? 0 : (it >= a.N) + (it >= 2 * a.N), n = it - t * a.N;
+        float acc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const QW& m = a.m[MODE == SWIGLU ? r : t];
+            const __amdgpu_buffer_rsrc_t rw = make_rsrc(m.w + static_cast<size_t>(n) * a.ws, a.ws * 4);
+            const __amdgpu_buffer_rsrc_t rz = make_rsrc(m.z + static_cast<size_t>(n) * a.zs, a.zs * 4);
+            const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.s + static_cast<size_t>(n) * a.ss, a.ss * 2);
+            float s = 0.0f;
+            for (int c0 = 0; c0 < nchunks; c0 += 64) {
+                const int c = c0 + lane; // beyond nchunks the buffer reads 0, the LDS index is clamped
+                const u32x4 w4 = __builtin_amdgcn_raw_buffer_load_b128(rw, c * 16, 0, kAuxStream);
+                const uint32_t zw = __builtin_amdgcn_raw_buffer_load_b32(rz, (c >> 5) * 4, 0, 0);
+                const uint16_t sb = __builtin_amdgcn_raw_buffer_load_b16(rs, (c >> 2) * 2, 0, 0);
+                const int cc = c < nchunks ? c : nchunks - 1;
+                float a0 = 0.0f, a1 = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const u32x4 xv = xs_dyn[i * nchunks + cc];
+                    const uint32_t w = w4[i], w8 = w >> 8;
+                    a0 = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[0]), a0, false);
+                    a1 = __builtin_amdgcn_fdot2(as_h2(w & 0x00F000F0u), as_h2(xv[1]), a1, false);
+                    a0 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[2]), a0, false);
+                    a1 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), as_h2(xv[3]), a1, false);
+                }
+                const float zf = static_cast<float>((zw >> zshift) & 0xFu);
+                float tt = a0 * 16777216.0f;
+                tt = fmaf(a1, 1048576.0f, tt);
+                tt = fmaf(-zf, c < nchunks ? sx[cc] : 0.0f, tt);
+                s = fmaf(tt, half_bits_to_float(sb), s);
+            }
+            acc[r] = wave_sum(s);
+        }
+        if (lane == 0) {
+            float v = acc[0];
+            if (MODE == SWIGLU) {
+                v *= 1.0f / (1.0f + expf(-v));
+                v *= acc[R - 1];
+            } else if (MODE == RESIDUAL) {
+                v += half_bits_to_float(a.out[t][n]);
+            }
+            a.out[t][n] = float_to_half_bits(v);
+        }
+    }
+}
+
+template <int J, int MODE, int STAGE>
+inline void launch_j(const Int4Args& a, int max_waves)
+{
+    const int nitems = MODE == QKV_ROPE ? 3 * (a.N / 2) : a.n_tensors * a.N;
+    const int waves = nitems < max_waves ? nitems : max_waves;
+    hipLaunchKernelGGL((int4_matvec_kernel<J, MODE, STAGE>), dim3(ceil_div(waves, 4)), dim3(256), 0, ctx().stream, a);
+}
+
+// Number of chunk-columns a lane holds per row for a K-input tensor.
+inline int chunk_columns(int ws) { return ceil_div(ws / 4, 64); }
+constexpr int kMaxChunkColumns = 8; // K <= 16384 on the unrolled kernels
+
+// Wavefronts kept resident per launch: 16 per CU while a lane holds up to 3
+// chunks of a row, 8 per CU for longer rows (more bytes in flight per lane).
+template <int MODE, int STAGE>
+inline int launch_int4(const char* fn, const Int4Args& a)
+{
+    const int J = chunk_columns(a.ws);
+    const int cus = ctx().num_cus > 0 ? ctx().num_cus : 256;
+    switch (J) {
+    case 1: launch_j<1, MODE, STAGE>(a, cus * 16); break;
+    case 2: launch_j<2, MODE, STAGE>(a, cus * 16); break;
+    case 3: launch_j<3, MODE, STAGE>(a, cus * 16); break;
+    case 4: launch_j<4, MODE, STAGE>(a, cus * 8); break;
+    case 5: launch_j<5, MODE, STAGE>(a, cus * 8); break;
+    case 6: launch_j<6, MODE, STAGE>(a, cus * 8); break;
+    case 7: launch_j<7, MODE, STAGE>(a, cus * 8); break;
+    case 8: launch_j<8, MODE, STAGE>(a, cus * 8); break;
+    default: {
+        if (MODE == QKV_ROPE || STAGE != STAGE_X)
+            return fail(LLAMA2_ERR_UNSUPPORTED, "%s: rows=%d exceeds the fused kernels' limit of %d", fn, a.K,
+                        kMaxChunkColumns * 2048);
+        const int nitems = a.n_tensors * a.N;
+        const int grid = ceil_div(nitems < cus * 8 ? nitems : cus * 8, 4);
+        constexpr int GM = (MODE == QKV_ROPE) ? PLAIN : MODE;
+        hipLaunchKernelGGL((int4_matvec_generic_kernel<GM>), dim3(grid), dim3(256),
+                           static_cast<size_t>(a.ws / 4) * 68, ctx().stream, a);
+    }
+    }
+    L2_LAUNCH_CHECK(fn);
+    return LLAMA2_OK;
+}
+
+} // namespace l2

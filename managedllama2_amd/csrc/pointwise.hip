@@ -55,6 +55,26 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_kernel(uint16_t* out, const ui
         out[i] = float_to_half_bits(rms * half_bits_to_float(gamma[i]) * half_bits_to_float(x[i]));
 }
 
+// The same module for sizes that are multiples of 8 up to 16384: 256 threads,
+// 16-byte accesses, and exactly the arithmetic (order included) that the fused
+// decode kernels apply while staging their input, so both paths agree bit for bit.
+template <int J>
+__global__ __launch_bounds__(256) void rmsnorm_vec_kernel(uint16_t* out, const uint16_t* x, const uint16_t* gamma,
+                                                          int size, float eps)
+{
+    __shared__ float red4[4];
+    VecPieces<J> xp, gp;
+    xp.load(x, size);
+    gp.load(gamma, size);
+    const float ss = block256_sum(xp.sum_squares(), red4);
+    const float rms = 1.0f / sqrtf(ss / static_cast<float>(size) + eps);
+    xp.scale(rms, gp);
+    const __amdgpu_buffer_rsrc_t ro = make_rsrc(out, size * 2);
+#pragma unroll
+    for (int i = 0; i < J; ++i) // pieces beyond `size` fall outside the buffer and are dropped
+        __builtin_amdgcn_raw_buffer_store_b128(xp.v[i], ro, (threadIdx.x + i * 256) * 16, 0, 0);
+}
+
 // One workgroup per head, one thread per rotated pair (t, t + head_size/2):
 // native/rope_kernel.cu:3-26.
 __global__ void rope_kernel(uint16_t* q, uint16_t* k, int n_kv_heads, int head_size, int pos, float theta)
@@ -177,7 +197,21 @@ int llama2_rmsnorm(llama2_half* output, const llama2_half* input, const llama2_h
     L2_REQUIRE_INIT();
     L2_CHECK(output && input && gamma, "llama2_rmsnorm: null pointer");
     L2_CHECK(size > 0, "llama2_rmsnorm: size=%d must be positive", size);
-    hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(kBlock), 0, ctx().stream, output, input, gamma, size, eps);
+    const int J = ceil_div(size, 2048);
+    if (size % 8 == 0 && J <= 8 && aligned(output, 16) && aligned(input, 16) && aligned(gamma, 16)) {
+#define L2_RMS_CASE(j)                                                                                           \
+    case j:                                                                                                      \
+        hipLaunchKernelGGL(rmsnorm_vec_kernel<j>, dim3(1), dim3(256), 0, ctx().stream, output, input, gamma, size, \
+                           eps);                                                                                 \
+        break;
+        switch (J) {
+            L2_RMS_CASE(1) L2_RMS_CASE(2) L2_RMS_CASE(3) L2_RMS_CASE(4) L2_RMS_CASE(5) L2_RMS_CASE(6) L2_RMS_CASE(7)
+            L2_RMS_CASE(8)
+        }
+#undef L2_RMS_CASE
+    } else {
+        hipLaunchKernelGGL(rmsnorm_kernel, dim3(1), dim3(kBlock), 0, ctx().stream, output, input, gamma, size, eps);
+    }
     L2_LAUNCH_CHECK("llama2_rmsnorm");
     return LLAMA2_OK;
 }

@@ -19,8 +19,11 @@ pytestmark = pytest.mark.gpu
 # Module outputs are rounded to fp16 between modules on both sides; a rounding that
 # falls the other way perturbs everything downstream by about one fp16 step of a
 # typical activation.  Whole-step logits are therefore compared norm-wise:
-# max|y - y*| <= LOGIT_TOL * max|y*|.
-LOGIT_TOL = 4e-3
+# max|y - y*| <= LOGIT_TOL * max|y*|.  With random int4 weights every layer
+# amplifies such a flip (measured: 1e-3 .. 5e-3 at the logits after three layers, the
+# same for the module-by-module and the fused launch sequence); single modules are
+# held to 2e-3 element-wise in their own tests.
+LOGIT_TOL = 1e-2
 
 SMALL = dict(dim=256, hidden_dim=640, n_layers=3, n_heads=2, n_kv_heads=2, vocab_size=1000, seq_len=48,
              rope_theta=10000.0)
@@ -68,6 +71,83 @@ def test_small_model_host_loop_and_decoder_agree(oracle):
     assert e1 >= len(g1) - 1  # at most one near-tie flip against the oracle
 
 
+FUSED = capi.DECODE_FUSED
+FUSED_GRAPH = capi.DECODE_FUSED | capi.DECODE_GRAPH
+# head_size must be 128 for the fused step
+HS128 = dict(dim=512, hidden_dim=1408, n_layers=3, n_heads=4, n_kv_heads=4, vocab_size=1000, seq_len=300,
+             rope_theta=10000.0)
+
+
+@pytest.mark.parametrize("mode", [FUSED, FUSED_GRAPH])
+def test_fused_step_against_oracle(oracle, mode):
+    model = synth.random_model(HS128, seed=8, rms_random=True)
+    exact, gen, _ = run_and_check(oracle, HS128, model, mode, n_prompt=4, steps=24, seed=404)
+    assert exact >= len(gen) - 1
+
+
+def test_fused_step_tracks_module_step(oracle):
+    """Same model, same prompt: the fused launches and the module-by-module
+    launches share the mat-vec, RMSNorm and RoPE arithmetic; only attention is
+    evaluated differently (block-wise softmax statistics), so logits agree to
+    well below the oracle tolerance."""
+    model = synth.random_model(HS128, seed=8, rms_random=True)
+    rng = synth.rng_for(405)
+    prompt = rng.integers(3, HS128["vocab_size"], 150).astype(np.int32)  # forces 2 attention blocks
+    outs = []
+    for mode in (capi.DECODE_MODULES, FUSED, FUSED_GRAPH):
+        t = Transformer(dict(HS128), model, mode=mode)
+        t.runstate.tokens.copy_to_device(prompt)
+        for pos in range(140):
+            t.Forward(pos, pos + 1)
+        outs.append((t.runstate.logits.to_host().astype(np.float64), t.runstate.keyCache.to_host(140 * 512)))
+        t.close()
+    assert np.array_equal(outs[1][0], outs[2][0])  # graph replay == eager launches, bit for bit
+    assert_close_normwise(outs[1][0], outs[0][0], "fused vs modules logits", 2e-3)
+    assert_close_normwise(outs[1][1].astype(np.float64), outs[0][1].astype(np.float64), "fused vs modules K cache", 2e-3)
+
+
+def test_graph_replays_are_stable(oracle):
+    """Replay the captured step several times with eager work and synchronisation
+    in between; every replay of the same position must reproduce the eager result."""
+    model = synth.random_model(HS128, seed=9)
+    rng = synth.rng_for(406)
+    prompt = rng.integers(3, HS128["vocab_size"], 8).astype(np.int32)
+    eager = Transformer(dict(HS128), model, mode=FUSED)
+    graph = Transformer(dict(HS128), model, mode=FUSED_GRAPH)
+    for t in (eager, graph):
+        t.runstate.tokens.copy_to_device(prompt)
+    for pos in range(8):
+        eager.Forward(pos, pos + 1)
+        want = eager.runstate.logits.to_host()
+        for rep in range(3):
+            graph.Forward(pos, pos + 1)
+            got = graph.runstate.logits.to_host()  # synchronises
+            assert np.array_equal(got.view(np.uint16), want.view(np.uint16)), (pos, rep)
+            capi.call("llama2_memset", graph.runstate.logits.ptr, 0, 16)  # eager work between replays
+    eager.close()
+    graph.close()
+
+
+@pytest.mark.parametrize("mode", [FUSED, FUSED_GRAPH])
+def test_device_resident_loop(oracle, mode):
+    model = synth.random_model(HS128, seed=10)
+    rng = synth.rng_for(407)
+    prompt = rng.integers(3, HS128["vocab_size"], 5).astype(np.int32)
+    ref = Transformer(dict(HS128), model, mode=mode)
+    want = list(ref.Generate(prompt, 40, stop_on_special=False))
+    t = Transformer(dict(HS128), model, mode=mode)
+    t.runstate.tokens.copy_to_device(prompt)
+    capi.call("llama2_decode_run", t._decoder, 0, 40, len(prompt))
+    got = list(t.runstate.tokens.to_host(41)[1:])
+    assert got == want
+    # continue from where it stopped
+    capi.call("llama2_decode_run", t._decoder, 40, 10, len(prompt))
+    more = list(ref.Generate(list(prompt), 50, stop_on_special=False))
+    assert list(t.runstate.tokens.to_host(51)[1:]) == more
+    ref.close()
+    t.close()
+
+
 def test_generate_matches_stepwise(oracle):
     model = synth.random_model(SMALL, seed=6)
     rng = synth.rng_for(402)
@@ -86,11 +166,12 @@ def test_generate_matches_stepwise(oracle):
     t2.close()
 
 
-def test_llama7b_shaped_layers(oracle):
+@pytest.mark.parametrize("mode", [capi.DECODE_MODULES, capi.DECODE_FUSED | capi.DECODE_GRAPH])
+def test_llama7b_shaped_layers(oracle, mode):
     """Real 7B tensor shapes (dim 4096, hidden 11008, 32 heads, vocab 32000), two layers."""
     cfg = dict(synth.LLAMA2_7B, n_layers=2, seq_len=32)
     model = synth.random_model(cfg, seed=7)
-    exact, gen, _ = run_and_check(oracle, cfg, model, capi.DECODE_MODULES, n_prompt=3, steps=6, seed=403)
+    exact, gen, _ = run_and_check(oracle, cfg, model, mode, n_prompt=3, steps=6, seed=403)
     assert exact >= len(gen) - 1
 
 
