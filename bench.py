@@ -4,16 +4,21 @@
 A "step" is one Llama-2-7B decoder layer's int4 mat-vec set at batch 1 (fused
 QKV 3x4096x4096, o-proj 4096x4096 + residual, fused SwiGLU gate/up
 2x11008x4096, down-proj 4096x11008 + residual): four launches through the C
-ABI.  Steps cycle through 32 distinct layers of weights (3.36 GB), so every
-step streams its 105 MB from HBM and not from the 256 MB Infinity Cache.
+ABI.  Steps cycle through the 32 distinct layers of a random-init 7B model
+(3.36 GB of int4 weights), so every step streams its 105 MB from HBM and not
+from the 256 MB Infinity Cache.  Launches are replayed from a captured
+hipGraph so the host's per-call cost never bounds what the GPU does.
 
 Prints ONE JSON line: whole-job HBM GB/s over the algorithmic bytes of the
-mat-vec set, the roofline record of the dominant kernel (fused SwiGLU), and
-the reference's single-threaded C# CPU path (restated in C) timed beside it.
+mat-vec set (`value`), the roofline record of the dominant kernel (fused
+SwiGLU), decode attention GB/s at 512/2048/4096 rows, full greedy decode
+tokens/s (128-token prompt + 256 generated tokens), and the reference's
+single-threaded C# CPU path (restated in C) timed beside it.
 """
 import argparse
 import ctypes as C
 import json
+import math
 import os
 import sys
 import time
@@ -52,36 +57,49 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3200)
     ap.add_argument("--warmup", type=int, default=320)
-    ap.add_argument("--layers", type=int, default=32, help="distinct weight copies cycled through")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
-    ap.add_argument("--only", default="", help="comma list of legs to run: set,kernel,cpu (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs: set,kernel,attn,decode,cpu (default all)")
+    ap.add_argument("--decode-mode", default="fused_graph", choices=["modules", "fused", "fused_graph"])
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (batch-1 decode has no cross-GPU exchange to measure); "
             "--gpus %d is not supported" % args.gpus)
         sys.exit(2)
-    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "cpu"}
+    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "attn", "decode", "cpu"}
 
     from managedllama2_amd import capi, synth
-    from managedllama2_amd.device import DeviceVariable, QWeight, init
+    from managedllama2_amd.device import DeviceVariable, init
+    from managedllama2_amd.transformer import Transformer
 
     init(0)
-    dim, hidden = 4096, 11008
+    cfg = dict(synth.LLAMA2_7B)  # seq_len 4096: room for the attention leg
+    dim, hidden, n_layers = cfg["dim"], cfg["hidden_dim"], cfg["n_layers"]
     sizes = synth.layer_matvec_set_bytes(dim, hidden)
     zs, ss, ws = (lambda t: (t[2], t[1], t[0]))(synth.qweight_sizes(dim))
     hzs, hss, hws = (lambda t: (t[2], t[1], t[0]))(synth.qweight_sizes(hidden))
 
+    # ---- the random-init 7B model (configs[4] distributions), generated layer by layer
     t0 = time.time()
     rng = synth.rng_for(1, 7)
-    host_layers = []
-    layers = []
-    for l in range(args.layers):
-        hl = synth.random_layer(rng, dim, hidden)
-        if l == 0:
-            host_layers.append(hl)  # kept for the CPU baseline
-        layers.append({k: QWeight.from_host(*hl[k]) for k in ("q", "k", "v", "o", "gate", "up", "down")})
-    log("generated + uploaded %d layers (%.2f GB) in %.1f s" %
-        (args.layers, args.layers * (sizes["total"] - 126_000) / 1e9, time.time() - t0))
+    first_layer = []
+
+    def lazy_layers():
+        for l in range(n_layers):
+            hl = synth.random_layer(rng, dim, hidden)
+            if l == 0:
+                first_layer.append(hl)  # kept on the host for the CPU baseline
+            yield hl
+
+    host = {"embedding": synth.normal_f16(rng, cfg["vocab_size"] * dim, 0.02),
+            "classifier": synth.normal_f16(rng, cfg["vocab_size"] * dim, 0.02),
+            "rms_final": np.ones(dim, np.float16), "layers": lazy_layers()}
+    mode = {"modules": capi.DECODE_MODULES, "fused": capi.DECODE_FUSED,
+            "fused_graph": capi.DECODE_FUSED | capi.DECODE_GRAPH}[args.decode_mode]
+    model = Transformer(cfg, host, mode=mode)
+    del host
+    layers = model.weights.layers
+    log("generated + uploaded the 7B model (%.2f GB of int4 layers) in %.1f s" %
+        (n_layers * (sizes["total"] - 126_000) / 1e9, time.time() - t0))
 
     xb_host = synth.normal_f16(rng, dim)
     xb = DeviceVariable.from_host(xb_host)
@@ -93,25 +111,28 @@ def main():
 
     def qkv(L):
         capi.call("llama2_qkv_mat_vec", q.ptr, kc.ptr, vc.ptr, xb.ptr,
-                  L["q"].Weight.ptr, L["q"].Zeros.ptr, L["q"].Scales.ptr,
-                  L["k"].Weight.ptr, L["k"].Zeros.ptr, L["k"].Scales.ptr,
-                  L["v"].Weight.ptr, L["v"].Zeros.ptr, L["v"].Scales.ptr, dim, dim, zs, ss, ws)
+                  L.queryWeight.Weight.ptr, L.queryWeight.Zeros.ptr, L.queryWeight.Scales.ptr,
+                  L.keyWeight.Weight.ptr, L.keyWeight.Zeros.ptr, L.keyWeight.Scales.ptr,
+                  L.valueWeight.Weight.ptr, L.valueWeight.Zeros.ptr, L.valueWeight.Scales.ptr,
+                  dim, dim, zs, ss, ws)
 
     def oproj(L):
-        capi.call("llama2_mat_vec_residual_int4", x.ptr, xb.ptr, L["o"].Weight.ptr, L["o"].Zeros.ptr,
-                  L["o"].Scales.ptr, dim, dim, zs, ss, ws)
+        w = L.outputWeight
+        capi.call("llama2_mat_vec_residual_int4", x.ptr, xb.ptr, w.Weight.ptr, w.Zeros.ptr, w.Scales.ptr,
+                  dim, dim, zs, ss, ws)
 
     def swiglu(L):
-        capi.call("llama2_mat_vec_swiglu", h.ptr, xb.ptr, L["gate"].Weight.ptr, L["gate"].Zeros.ptr,
-                  L["gate"].Scales.ptr, L["up"].Weight.ptr, L["up"].Zeros.ptr, L["up"].Scales.ptr,
-                  dim, hidden, zs, ss, ws)
+        g, u = L.gateWeight, L.upWeight
+        capi.call("llama2_mat_vec_swiglu", h.ptr, xb.ptr, g.Weight.ptr, g.Zeros.ptr, g.Scales.ptr,
+                  u.Weight.ptr, u.Zeros.ptr, u.Scales.ptr, dim, hidden, zs, ss, ws)
 
     def down(L):
-        capi.call("llama2_mat_vec_residual_int4", x.ptr, h.ptr, L["down"].Weight.ptr, L["down"].Zeros.ptr,
-                  L["down"].Scales.ptr, hidden, dim, hzs, hss, hws)
+        w = L.downWeight
+        capi.call("llama2_mat_vec_residual_int4", x.ptr, h.ptr, w.Weight.ptr, w.Zeros.ptr, w.Scales.ptr,
+                  hidden, dim, hzs, hss, hws)
 
     def step(i):
-        L = layers[i % len(layers)]
+        L = layers[i % n_layers]
         qkv(L)
         oproj(L)
         swiglu(L)
@@ -120,8 +141,7 @@ def main():
     ev = Events(capi)
 
     def capture(fn, n):
-        """Record n calls of fn(i) into one hipGraph (one submission per replay,
-        so the host's per-call cost never bounds what the GPU is seen to do)."""
+        """Record n calls of fn(i) into one hipGraph."""
         g = C.c_void_p()
         capi.call("llama2_graph_begin_capture")
         for i in range(n):
@@ -137,59 +157,151 @@ def main():
         ms = ev.stop_ms()
         capi.call("llama2_sync")
         return ms
+
     result = {
         "metric": "int4 mat-vec HBM GB/s, Llama-2-7B decoder-layer mat-vec set, batch 1",
         "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int4 weights x f16 activations, f32 accumulate",
-        "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights x f16 activations, f32 accumulate", "data": "synthetic",
         "config": {"workload": "configs[1]: 7B layer mat-vec set (QKV, o+res, SwiGLU, down+res), "
-                               "%d distinct weight copies cycled (cold HBM)" % args.layers,
+                               "%d distinct layers cycled (cold HBM)" % n_layers,
                    "dim": dim, "hidden_dim": hidden, "algorithmic_bytes_per_step": sizes["total"]},
     }
 
-    cycle = len(layers)
     if "set" in legs:
-        # one graph = one pass over all distinct layers; K steps = K/cycle replays
-        graph = capture(step, cycle)
-        replays = max(args.steps // cycle, 1)
-        args.steps = replays * cycle
-        for _ in range(max(args.warmup // cycle, 1)):
+        # one graph = one pass over all distinct layers; K steps = K / n_layers replays
+        graph = capture(step, n_layers)
+        replays = max(args.steps // n_layers, 1)
+        steps = replays * n_layers
+        for _ in range(max(args.warmup // n_layers, 1)):
             capi.call("llama2_graph_launch", graph)
         capi.call("llama2_sync")
         wall0 = time.perf_counter()
         ms = timed_replays(graph, replays)
         wall = time.perf_counter() - wall0
         capi.call("llama2_graph_destroy", graph)
-        result["steps"] = args.steps
-        ms_per_step = ms / args.steps
+        ms_per_step = ms / steps
         gbps = sizes["total"] / (ms_per_step * 1e-3) / 1e9
-        result.update(value=round(gbps, 1), ms_per_step=round(ms_per_step, 5),
+        result.update(steps=steps, value=round(gbps, 1), ms_per_step=round(ms_per_step, 5),
                       pct_of_hbm_peak=round(100 * gbps / HBM_PEAK_GBPS, 2),
-                      wall_ms_per_step=round(1e3 * wall / args.steps, 5))
+                      wall_ms_per_step=round(1e3 * wall / steps, 5))
         log("layer mat-vec set: %.2f us/step, %.0f GB/s (%.1f%% of 8 TB/s)" %
             (1e3 * ms_per_step, gbps, 100 * gbps / HBM_PEAK_GBPS))
 
     if "kernel" in legs:
         per_kernel = {}
         for name, fn in (("qkv", qkv), ("o", oproj), ("swiglu", swiglu), ("down", down)):
-            graph = capture(lambda i, fn=fn: fn(layers[i % cycle]), cycle)
-            replays = max(args.steps // cycle // 2, 2)
+            graph = capture(lambda i, fn=fn: fn(layers[i % n_layers]), n_layers)
+            replays = max(args.steps // n_layers // 2, 2)
             capi.call("llama2_graph_launch", graph)
-            us = 1e3 * timed_replays(graph, replays) / (replays * cycle)
+            us = 1e3 * timed_replays(graph, replays) / (replays * n_layers)
             capi.call("llama2_graph_destroy", graph)
             per_kernel[name] = {"us": round(us, 3), "GBps": round(sizes[name] / us / 1e3, 1),
                                 "bytes": sizes[name]}
             log("  %-7s %8.2f us  %7.0f GB/s  (%d B)" % (name, us, sizes[name] / us / 1e3, sizes[name]))
         dom = per_kernel["swiglu"]
-        result["roofline"] = {"bound": "hbm", "kernel": "int4_swiglu_kernel (fused gate/up, 2x11008x4096)",
+        result["roofline"] = {"bound": "hbm", "kernel": "int4_matvec_kernel<2, SWIGLU> (fused gate/up, 2x11008x4096)",
                               "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                               "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
                               "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_us": dom["us"]}
         result["per_kernel"] = per_kernel
 
+    if "calib" in legs:
+        # a plain copy of known size: what FETCH_SIZE / WRITE_SIZE read for it scales the counters
+        # of the mat-vec kernels (rocprofv3 --pmc runs, see profiles/)
+        n = 1 << 30
+        src, dst = DeviceVariable.zeros(np.uint8, n), DeviceVariable.zeros(np.uint8, n)
+        capi.call("llama2_sync")
+        ev.start()
+        for _ in range(4):
+            capi.call("llama2_memcpy_d2d", dst.ptr, src.ptr, n)
+        ms = ev.stop_ms() / 4
+        result["copy_calibration"] = {"bytes_read": n, "bytes_written": n, "us": round(1e3 * ms, 1),
+                                      "GBps_read_plus_write": round(2 * n / ms / 1e6, 1)}
+        log("copy calibration: 1 GiB -> 1 GiB in %.1f us (%.0f GB/s read+write)" % (1e3 * ms, 2 * n / ms / 1e6))
+        src.free()
+        dst.free()
+
+    if "attn" in legs:
+        # configs[3]: decode attention over the fp16 KV cache, 32 heads x 128, RoPE at pos = S on the
+        # newest row, scores, softmax, weighted value sum; cycled over the 32 layers' cache slices
+        rs = model.runstate
+        seq_cap = model.config.seq_len
+        kv_bytes = rs.keyCache.nbytes
+        fill = synth.normal_f16(synth.rng_for(3), 1 << 22)
+        for off in range(0, kv_bytes // 2, fill.size):  # N(0,1) values everywhere
+            n = min(fill.size, kv_bytes // 2 - off)
+            rs.keyCache.copy_to_device(fill[:n], off)
+            rs.valueCache.copy_to_device(fill[:n], off)
+        rs.q.copy_to_device(synth.normal_f16(synth.rng_for(4), dim))
+        hs, heads = dim // cfg["n_heads"], cfg["n_heads"]
+        scale = 1.0 / math.sqrt(hs)
+        attn = {}
+        for S in (512, 2048, 4096):
+            if S > seq_cap:
+                continue
+            nbytes = 2 * S * dim * 2 + 2 * dim * 2
+
+            def modules(i, S=S):
+                lo = (i % n_layers) * seq_cap * dim
+                capi.call("llama2_rope", rs.q.ptr, rs.keyCache.offset_pointer(lo + (S - 1) * dim), heads, hs, S,
+                          10000.0, heads)
+                capi.call("llama2_mat_vec_strided", rs.attention.ptr, rs.q.ptr, rs.keyCache.offset_pointer(lo),
+                          hs, S, hs, hs, dim, S, scale, heads)
+                capi.call("llama2_softmax", rs.attention.ptr, S, heads)
+                capi.call("llama2_vec_mat", rs.xb.ptr, rs.attention.ptr, rs.valueCache.offset_pointer(lo),
+                          hs, S, hs, hs, dim, heads)
+
+            def fused(i, S=S):
+                lo = (i % n_layers) * seq_cap * dim
+                capi.call("llama2_rope", rs.q.ptr, rs.keyCache.offset_pointer(lo + (S - 1) * dim), heads, hs, S,
+                          10000.0, heads)
+                capi.call("llama2_multi_head_attention", rs.xb.ptr, rs.q.ptr, rs.keyCache.offset_pointer(lo),
+                          rs.valueCache.offset_pointer(lo), hs, dim, S, scale, heads)
+
+            row = {"bytes": nbytes}
+            for name, fn in (("modules", modules), ("fused", fused)):
+                fn(0)  # sizes the library's scratch before capture
+                graph = capture(fn, n_layers)
+                capi.call("llama2_graph_launch", graph)
+                us = 1e3 * timed_replays(graph, 10) / (10 * n_layers)
+                capi.call("llama2_graph_destroy", graph)
+                row[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)}
+            attn["S=%d" % S] = row
+            log("  attention S=%-5d rope+scores+softmax+vecmat %7.2f us %6.0f GB/s | rope+fused %7.2f us %6.0f GB/s" %
+                (S, row["modules"]["us"], row["modules"]["GBps"], row["fused"]["us"], row["fused"]["GBps"]))
+        result["attention"] = attn
+
+    if "decode" in legs:
+        # configs[4]: 128 seeded prompt tokens, 256 greedy tokens, every step on the device
+        n_prompt, n_gen = 128, 256
+        steps = n_prompt + n_gen - 1
+        prompt = synth.rng_for(5).integers(3, cfg["vocab_size"], n_prompt).astype(np.int32)
+        model.runstate.tokens.copy_to_device(prompt)
+        capi.call("llama2_decode_run", model._decoder, 0, 16, n_prompt)  # warm-up
+        capi.call("llama2_sync")
+        ev.start()
+        capi.call("llama2_decode_run", model._decoder, 0, steps, n_prompt)
+        ms = ev.stop_ms()
+        toks = model.runstate.tokens.to_host(n_prompt + n_gen)
+        tok_s = steps / (ms * 1e-3)
+        kv_avg = 2 * n_layers * (steps + 1) / 2 * dim * 2
+        bytes_tok = (n_layers * (sizes["total"] - 126_000 + 2 * 2 * dim) + 2 * cfg["vocab_size"] * dim
+                     + 2 * dim + 2 * dim + kv_avg)
+        result["decode"] = {"tokens_per_s": round(tok_s, 1), "ms_per_token": round(ms / steps, 4),
+                            "forward_steps": steps, "prompt": n_prompt, "generated": n_gen,
+                            "mode": args.decode_mode,
+                            "GBps": round(bytes_tok * tok_s / 1e9, 1),
+                            "pct_of_hbm_peak": round(100 * bytes_tok * tok_s / 1e9 / HBM_PEAK_GBPS, 2),
+                            "bandwidth_bound_tokens_per_s": round(HBM_PEAK_GBPS * 1e9 / bytes_tok, 1),
+                            "last_tokens": [int(t) for t in toks[-4:]]}
+        log("decode: %.1f tok/s (%.3f ms/token, %.0f GB/s = %.1f%% of peak; ceiling %.0f tok/s)" %
+            (tok_s, ms / steps, bytes_tok * tok_s / 1e9, 100 * bytes_tok * tok_s / 1e9 / HBM_PEAK_GBPS,
+             HBM_PEAK_GBPS * 1e9 / bytes_tok))
+
     if "cpu" in legs and args.cpu_seconds > 0:
         from oracle import oracle
-        hm_layer = host_layers[0]
+        hm_layer = first_layer[0]
         lp = oracle.LayerPtr()
         for name in ("q", "k", "v", "o", "gate", "up", "down"):
             W, Z, S = hm_layer[name]
@@ -209,6 +321,7 @@ def main():
                                   "seconds_per_step": round(spent / n_sets, 3), "host_cpus": os.cpu_count()}
         log("cpu baseline: %.3f s per layer set on 1 core (%.4f GB/s)" % (spent / n_sets, cpu_gbps))
 
+    model.close()
     print(json.dumps(result), flush=True)
 
 

@@ -69,6 +69,9 @@ int llama2_memcpy_h2d(void* dst, size_t dst_offset_bytes, const void* src, size_
 /* explicit CudaDeviceVariable<T> -> T[] and the 1-element indexer read
  * `runstate.tokens[nextPosition]` (src/Sampler.cs:69).  Waits for the stream. */
 int llama2_memcpy_d2h(void* dst, const void* src, size_t src_offset_bytes, size_t bytes);
+/* CudaDeviceVariable.CopyToDevice(CudaDeviceVariable): asynchronous device-to-
+ * device copy by a plain copy kernel (16-byte granularity, no overlap). */
+int llama2_memcpy_d2d(void* dst, const void* src, size_t bytes);
 /* Asynchronous fill (tests and RunState set-up; ManagedCuda's Memset). */
 int llama2_memset(void* dst, int byte_value, size_t bytes);
 /* CudaContext.GetFreeDeviceMemorySize(): src/RunState.cs:34. */
@@ -171,6 +174,18 @@ int llama2_mat_vec_strided(llama2_half* output, const llama2_half* vector,
 int llama2_vec_mat(llama2_half* output, const llama2_half* vector, const llama2_half* matrix,
                    int rows, int cols, int m_col_stride, int o_stride, int m_row_stride,
                    int n_heads);
+
+/* Transformer.MultiHeadAttention (src/Transformer.cs:150-156) as ONE launch:
+ * scores over `seq_length` rows of `key`, softmax, weighted sum of `value`
+ * rows, without the round trip through the `attention` scratch.  key / value
+ * are the cache slices of the layer (caller adds layerOffset), rows of `dim`
+ * halfs; head h uses columns h*head_size .. of q, key, value and output.
+ * Scores are rounded to fp16 as the reference's attention buffer does.
+ * head_size must be 128; other sizes: LLAMA2_ERR_UNSUPPORTED, use the three
+ * modules above. */
+int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, const llama2_half* key,
+                                const llama2_half* value, int head_size, int dim, int seq_length,
+                                float scale, int n_heads);
 
 /* ------------------------------------------------------- pointwise modules */
 

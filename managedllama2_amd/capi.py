@@ -71,6 +71,7 @@ _SIGNATURES = {
     "llama2_free": [vp],
     "llama2_memcpy_h2d": [vp, sz, vp, sz],
     "llama2_memcpy_d2h": [vp, vp, sz, sz],
+    "llama2_memcpy_d2d": [vp, vp, sz],
     "llama2_memset": [vp, i, sz],
     "llama2_mem_info": [C.POINTER(sz), C.POINTER(sz)],
     "llama2_sync": [],
@@ -89,6 +90,7 @@ _SIGNATURES = {
     "llama2_mat_vec": [vp, vp, vp, i, i],
     "llama2_mat_vec_strided": [vp, vp, vp, i, i, i, i, i, i, f, i],
     "llama2_vec_mat": [vp, vp, vp, i, i, i, i, i, i],
+    "llama2_multi_head_attention": [vp, vp, vp, vp, i, i, i, f, i],
     "llama2_rmsnorm": [vp, vp, vp, i, f],
     "llama2_rope": [vp, vp, i, i, i, f, i],
     "llama2_softmax": [vp, i, i],

@@ -22,7 +22,11 @@ struct Context {
     // fp32 partial sums of the sequence-split attention kernels
     float* attn_partials = nullptr;
     size_t attn_partials_bytes = 0;
+    // per-head arrival counters of llama2_multi_head_attention (zero between launches)
+    unsigned* attn_counters = nullptr;
 };
+
+constexpr int kMaxAttnHeads = 1024;
 
 Context& ctx();
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
@@ -130,6 +134,30 @@ __device__ __forceinline__ float wave_max(float v)
         v = fmaxf(v, __shfl_xor(v, off, 64));
     return v;
 }
+
+// Data handed from one workgroup to another INSIDE a kernel (attention partials,
+// arrival counters) moves through agent-scope accesses: the store is written
+// through to the level every XCD sees, the load bypasses this XCD's possibly
+// stale L2 lines.  That replaces __threadfence(), whose L2 write-back +
+// invalidate costs tens of microseconds on this part.  Ordering: a producer
+// calls wait_agent_stores() before it announces its data with an atomic.
+__device__ __forceinline__ void store_agent(float* p, float v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_agent(const float* p)
+{
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void store_agent(unsigned* p, unsigned v)
+{
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned add_agent(unsigned* p, unsigned v)
+{
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void wait_agent_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // Sum over a 256-thread workgroup (4 wavefronts), identical in every thread and
 // independent of which kernel calls it: RMSNorm is evaluated both by the

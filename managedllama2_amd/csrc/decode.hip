@@ -38,7 +38,8 @@ struct AttnArgs {
     uint16_t* out; // [n_heads * 128]
     float* part;   // [n_heads][max_splits][kPartStride]
     unsigned* counters; // [n_heads], zero between launches
-    const int* pos_ptr;
+    const int* pos_ptr; // device-resident position, or null: attend `seq` rows
+    int seq;
     int dim;
     int max_splits;
     float scale;
@@ -50,7 +51,7 @@ __global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
     __shared__ float red[16][kRopeHeadSize];
     __shared__ int is_last;
     const int split = blockIdx.x, h = blockIdx.y;
-    const int S = a.pos_ptr[0] + 1; // attends rows 0..pos (src/Transformer.cs:175)
+    const int S = a.pos_ptr ? a.pos_ptr[0] + 1 : a.seq; // attends rows 0..pos (src/Transformer.cs:175)
     const int nsplit = (S + kSplitT - 1) / kSplitT;
     if (split >= nsplit)
         return;
@@ -123,33 +124,30 @@ __global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
     }
     float* P = a.part + (static_cast<size_t>(h) * a.max_splits + split) * kPartStride;
     if (threadIdx.x < kRopeHeadSize)
-        P[threadIdx.x] = val;
+        store_agent(P + threadIdx.x, val);
     if (threadIdx.x == 0) {
-        P[kRopeHeadSize] = m;
-        P[kRopeHeadSize + 1] = l;
+        store_agent(P + kRopeHeadSize, m);
+        store_agent(P + kRopeHeadSize + 1, l);
     }
-    __threadfence(); // publish the partials before announcing them
+    wait_agent_stores(); // the partials are visible device-wide before they are announced
     __syncthreads();
-    if (threadIdx.x == 0) {
-        const unsigned prev = atomicAdd(&a.counters[h], 1u);
-        is_last = prev == static_cast<unsigned>(nsplit - 1);
-    }
+    if (threadIdx.x == 0)
+        is_last = add_agent(&a.counters[h], 1u) == static_cast<unsigned>(nsplit - 1);
     __syncthreads();
     if (!is_last)
         return;
-    __threadfence(); // see every other block's partials
     if (threadIdx.x == 0)
-        a.counters[h] = 0; // ready for the next launch
+        store_agent(&a.counters[h], 0u); // ready for the next launch
     if (threadIdx.x < kRopeHeadSize) {
         const float* P0 = a.part + static_cast<size_t>(h) * a.max_splits * kPartStride;
         float M = -INFINITY;
         for (int i = 0; i < nsplit; ++i)
-            M = fmaxf(M, P0[i * kPartStride + kRopeHeadSize]);
+            M = fmaxf(M, load_agent(P0 + i * kPartStride + kRopeHeadSize));
         float L = 0.0f, O = 0.0f;
         for (int i = 0; i < nsplit; ++i) {
-            const float w = expf(P0[i * kPartStride + kRopeHeadSize] - M);
-            L = fmaf(w, P0[i * kPartStride + kRopeHeadSize + 1], L);
-            O = fmaf(w, P0[i * kPartStride + threadIdx.x], O);
+            const float w = expf(load_agent(P0 + i * kPartStride + kRopeHeadSize) - M);
+            L = fmaf(w, load_agent(P0 + i * kPartStride + kRopeHeadSize + 1), L);
+            O = fmaf(w, load_agent(P0 + i * kPartStride + threadIdx.x), O);
         }
         out[threadIdx.x] = float_to_half_bits(O / L);
     }
@@ -416,6 +414,34 @@ void release(llama2_decoder* d)
 } // namespace
 
 extern "C" {
+
+int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, const llama2_half* key,
+                                const llama2_half* value, int head_size, int dim, int seq_length, float scale,
+                                int n_heads)
+{
+    L2_REQUIRE_INIT();
+    const char* fn = "llama2_multi_head_attention";
+    L2_CHECK(output && query && key && value, "%s: null pointer", fn);
+    L2_CHECK(seq_length > 0 && n_heads > 0 && dim > 0, "%s: seq_length=%d n_heads=%d dim=%d must be positive", fn,
+             seq_length, n_heads, dim);
+    if (head_size != kRopeHeadSize)
+        return fail(LLAMA2_ERR_UNSUPPORTED, "%s: head_size=%d, only 128 is implemented (use the three modules)", fn,
+                    head_size);
+    L2_CHECK(dim % 8 == 0 && dim >= n_heads * head_size, "%s: dim=%d must be a multiple of 8 and hold %d heads", fn, dim,
+             n_heads);
+    L2_CHECK(aligned(query, 16) && aligned(key, 16) && aligned(value, 16), "%s: q/k/v must be 16-byte aligned", fn);
+    L2_CHECK(n_heads <= kMaxAttnHeads, "%s: n_heads=%d exceeds %d", fn, n_heads, kMaxAttnHeads);
+    const int splits = ceil_div(seq_length, kSplitT);
+    if (splits > 1)
+        L2_TRY(ensure_attn_partials(sizeof(float) * static_cast<size_t>(n_heads) * splits * kPartStride));
+    AttnArgs a{};
+    a.q = query, a.kcache = key, a.vcache = value, a.out = output;
+    a.part = ctx().attn_partials, a.counters = ctx().attn_counters, a.pos_ptr = nullptr, a.seq = seq_length;
+    a.dim = dim, a.max_splits = splits, a.scale = scale;
+    hipLaunchKernelGGL(fused_attn_kernel, dim3(splits, n_heads), dim3(256), 0, ctx().stream, a);
+    L2_LAUNCH_CHECK(fn);
+    return LLAMA2_OK;
+}
 
 int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
                          const llama2_transformer_weights* weights, const llama2_run_state* state, int mode)

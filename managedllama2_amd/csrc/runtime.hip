@@ -77,6 +77,8 @@ int llama2_init(int device)
                     device, prop.gcnArchName);
     c.num_cus = prop.multiProcessorCount;
     L2_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
+    L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.attn_counters), kMaxAttnHeads * sizeof(unsigned)));
+    L2_HIP(hipMemset(c.attn_counters, 0, kMaxAttnHeads * sizeof(unsigned)));
     c.device = device;
     c.ready = true;
     g_err[0] = 0;
@@ -93,6 +95,9 @@ int llama2_shutdown(void)
         L2_HIP(hipFree(c.attn_partials));
     c.attn_partials = nullptr;
     c.attn_partials_bytes = 0;
+    if (c.attn_counters)
+        L2_HIP(hipFree(c.attn_counters));
+    c.attn_counters = nullptr;
     L2_HIP(hipStreamDestroy(c.stream));
     c.stream = nullptr;
     c.ready = false;
@@ -176,6 +181,33 @@ int llama2_memset(void* dst, int byte_value, size_t bytes)
     hipLaunchKernelGGL(fill_bytes_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx().stream,
                        static_cast<uint8_t*>(dst), static_cast<uint8_t>(byte_value), bytes);
     L2_LAUNCH_CHECK("fill_bytes_kernel");
+    return LLAMA2_OK;
+}
+
+// Plain 16-byte-per-lane copy: every byte is read once and written once.
+__global__ __launch_bounds__(256) void copy_bytes_kernel(u32x4* dst, const u32x4* src, size_t n16)
+{
+    size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (; i < n16; i += stride)
+        dst[i] = src[i];
+}
+
+int llama2_memcpy_d2d(void* dst, const void* src, size_t bytes)
+{
+    L2_REQUIRE_INIT();
+    if (bytes == 0)
+        return LLAMA2_OK;
+    L2_CHECK(dst && src, "llama2_memcpy_d2d: null pointer");
+    L2_CHECK(aligned(dst, 16) && aligned(src, 16) && bytes % 16 == 0,
+             "llama2_memcpy_d2d: pointers and size must be multiples of 16 bytes");
+    L2_CHECK(!overlap(dst, bytes, src, bytes), "llama2_memcpy_d2d: ranges overlap");
+    size_t blocks = (bytes / 16 + 1023) / 1024;
+    if (blocks > 65536)
+        blocks = 65536;
+    hipLaunchKernelGGL(copy_bytes_kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ctx().stream,
+                       static_cast<u32x4*>(dst), static_cast<const u32x4*>(src), bytes / 16);
+    L2_LAUNCH_CHECK("copy_bytes_kernel");
     return LLAMA2_OK;
 }
 
