@@ -174,6 +174,10 @@ __device__ __forceinline__ float block256_sum(float v, float* lds4)
     return t;
 }
 
+// Cache-policy bits of the raw buffer load/store builtins on gfx94x/gfx950.
+constexpr int kAuxNonTemporal = 2; // "nt": streamed once, do not keep
+constexpr int kAuxAgent = 16;      // "sc1": coherent at agent scope (sees other workgroups' sc1 stores)
+
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* p, uint32_t bytes)
 {
     // raw buffer, 32-bit elements; out-of-range reads return 0

@@ -138,29 +138,70 @@ __global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
         return;
     if (threadIdx.x == 0)
         store_agent(&a.counters[h], 0u); // ready for the next launch
+    // Merge the blocks of this head.  The partials are read with agent-scope
+    // buffer loads (they were written by other workgroups of this launch); a read
+    // beyond the last block returns 0, so the loads are unconditional and many of
+    // them are in flight at once.
+    const __amdgpu_buffer_rsrc_t rp = make_rsrc(a.part + static_cast<size_t>(h) * a.max_splits * kPartStride,
+                                                static_cast<uint32_t>(nsplit) * kPartStride * sizeof(float));
+    float* wsh = sc;       // per-block weights exp(m_i - M)   (nsplit <= 64 <= kSplitT)
+    float* lsh = &red[0][0]; // the merged denominator
+    if (threadIdx.x < 64) { // one wavefront: block i in lane i
+        const int off = (threadIdx.x * kPartStride + kRopeHeadSize) * 4;
+        const bool have = static_cast<int>(threadIdx.x) < nsplit;
+        const float mi = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rp, off, 0, kAuxAgent));
+        const float li = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rp, off + 4, 0, kAuxAgent));
+        const float M = wave_max(have ? mi : -INFINITY);
+        const float w = have ? expf(mi - M) : 0.0f;
+        wsh[threadIdx.x] = w;
+        const float L = wave_sum(w * li);
+        if (threadIdx.x == 0)
+            lsh[0] = L;
+    }
+    __syncthreads();
     if (threadIdx.x < kRopeHeadSize) {
-        const float* P0 = a.part + static_cast<size_t>(h) * a.max_splits * kPartStride;
-        float M = -INFINITY;
-        for (int i = 0; i < nsplit; ++i)
-            M = fmaxf(M, load_agent(P0 + i * kPartStride + kRopeHeadSize));
-        float L = 0.0f, O = 0.0f;
-        for (int i = 0; i < nsplit; ++i) {
-            const float w = expf(load_agent(P0 + i * kPartStride + kRopeHeadSize) - M);
-            L = fmaf(w, load_agent(P0 + i * kPartStride + kRopeHeadSize + 1), L);
-            O = fmaf(w, load_agent(P0 + i * kPartStride + threadIdx.x), O);
+        float O = 0.0f;
+        for (int i0 = 0; i0 < nsplit; i0 += 8) { // block order is fixed: deterministic
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                v[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                     rp, ((i0 + u) * kPartStride + static_cast<int>(threadIdx.x)) * 4, 0,
+                                                     kAuxAgent));
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                O = fmaf(i0 + u < nsplit ? wsh[i0 + u] : 0.0f, v[u], O);
         }
-        out[threadIdx.x] = float_to_half_bits(O / L);
+        out[threadIdx.x] = float_to_half_bits(O / lsh[0]);
     }
 }
 
 // ---------------------------------------------------------------- step state
 // state[0] = position, state[1] = first position whose token is generated,
-// state[2] = 1 to advance the position after sampling.
-__global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance)
+// state[2] = 1 to advance the position after sampling; the 128 floats behind
+// the 4 ints hold (cos, sin) of the position's RoPE angles, so the 32 QKV
+// launches of a step do not each spend a microsecond in powf/sinf/cosf.
+constexpr int kStateInts = 4;
+constexpr size_t kStateBytes = kStateInts * sizeof(int) + kRopeHeadSize * sizeof(float);
+
+__device__ __forceinline__ void write_rope_table(int* state, int i, int pos, float theta)
 {
-    state[0] = pos;
-    state[1] = n_prompt;
-    state[2] = advance;
+    float c, s;
+    rope_cos_sin(c, s, i, kRopeHeadSize, pos, theta);
+    float* tab = reinterpret_cast<float*>(state + kStateInts);
+    tab[2 * i] = c;
+    tab[2 * i + 1] = s;
+}
+
+__global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance, float theta)
+{
+    if (threadIdx.x == 0) {
+        state[0] = pos;
+        state[1] = n_prompt;
+        state[2] = advance;
+    }
+    if (threadIdx.x < kRopeHeadSize / 2)
+        write_rope_table(state, threadIdx.x, pos, theta);
 }
 
 __device__ __forceinline__ bool better(float va, int ia, float vb, int ib)
@@ -170,13 +211,31 @@ __device__ __forceinline__ bool better(float va, int ia, float vb, int ib)
 
 // Sampler.Sample greedy branch (src/Sampler.cs:44-47) against the device state:
 // tokens[pos+1] = argmax(logits) iff pos+1 >= n_prompt; lowest index wins ties.
-__global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, int size, int* tokens, int* state)
+__global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, int size, int* tokens, int* state,
+                                                           float theta)
 {
     __shared__ float sv[16];
     __shared__ int si[16];
+    const int pos0 = state[0], advance0 = state[2]; // read by every thread before thread 0 updates them
+    if (advance0 && threadIdx.x >= 64 && threadIdx.x < 64 + kRopeHeadSize / 2)
+        write_rope_table(state, threadIdx.x - 64, pos0 + 1, theta); // for the next step
     float bv = -INFINITY;
     int bi = INT_MAX;
-    for (int i = threadIdx.x; i < size; i += 1024) {
+    // 16 bytes per load while whole groups of 8 remain (x is 16-byte aligned:
+    // checked on the host), the last size % 8 elements one by one
+    const int n8 = size >> 3;
+    for (int g = threadIdx.x; g < n8; g += 1024) {
+        const u32x4 v = reinterpret_cast<const u32x4*>(x)[g];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float f = half_bits_to_float(static_cast<uint16_t>(v[k >> 1] >> (16 * (k & 1))));
+            if (better(f, g * 8 + k, bv, bi)) {
+                bv = f;
+                bi = g * 8 + k;
+            }
+        }
+    }
+    for (int i = n8 * 8 + threadIdx.x; i < size; i += 1024) {
         const float f = half_bits_to_float(x[i]);
         if (better(f, i, bv, bi)) {
             bv = f;
@@ -210,11 +269,10 @@ __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, in
             }
         }
         if (threadIdx.x == 0) {
-            const int pos = state[0];
-            if (pos + 1 >= state[1])
-                tokens[pos + 1] = bi == INT_MAX ? 0 : bi;
-            if (state[2])
-                state[0] = pos + 1;
+            if (pos0 + 1 >= state[1])
+                tokens[pos0 + 1] = bi == INT_MAX ? 0 : bi;
+            if (advance0)
+                state[0] = pos0 + 1;
         }
     }
 }
@@ -321,6 +379,7 @@ int forward_fused(llama2_decoder* d)
                 a.embedding = d->w.token_embedding_table, a.tokens = s.tokens, a.vocab = c.vocab_size, a.x_out = s.x;
             a.pos_ptr = d->state;
             a.kv_dim = d->kv_dim, a.theta = c.rope_theta;
+            a.rope_table = reinterpret_cast<const float*>(d->state + kStateInts);
             L2_TRY((launch_int4<QKV_ROPE, STAGE_RMSNORM>("fused qkv", a)));
         }
         {
@@ -360,14 +419,15 @@ int forward_fused(llama2_decoder* d)
 int launch_argmax_step(llama2_decoder* d)
 {
     hipLaunchKernelGGL(argmax_step_kernel, dim3(1), dim3(1024), 0, ctx().stream, d->s.logits, d->cfg.vocab_size,
-                       d->s.tokens, d->state);
+                       d->s.tokens, d->state, d->cfg.rope_theta);
     L2_LAUNCH_CHECK("argmax_step_kernel");
     return LLAMA2_OK;
 }
 
 int set_state(llama2_decoder* d, int pos, int n_prompt, int advance)
 {
-    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(1), 0, ctx().stream, d->state, pos, n_prompt, advance);
+    hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, ctx().stream, d->state, pos, n_prompt, advance,
+                       d->cfg.rope_theta);
     L2_LAUNCH_CHECK("set_state_kernel");
     return LLAMA2_OK;
 }
@@ -499,7 +559,8 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
              "%s: null pointer in run state", fn);
     for (const void* p : {static_cast<const void*>(state->x), static_cast<const void*>(state->xb),
                           static_cast<const void*>(state->h), static_cast<const void*>(state->q),
-                          static_cast<const void*>(state->key_cache), static_cast<const void*>(state->value_cache)})
+                          static_cast<const void*>(state->key_cache), static_cast<const void*>(state->value_cache),
+                          static_cast<const void*>(state->logits)})
         L2_CHECK(aligned(p, 16), "%s: run-state buffers must be 16-byte aligned", fn);
     llama2_decoder* d = new (std::nothrow) llama2_decoder();
     L2_CHECK(d, "%s: out of host memory", fn);
@@ -513,7 +574,7 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     d->head_size = c.dim / c.n_heads;
     if (fused) {
         d->max_splits = ceil_div(c.seq_len, kSplitT);
-        hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->state), 4 * sizeof(int));
+        hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->state), kStateBytes);
         if (e == hipSuccess)
             e = hipMalloc(reinterpret_cast<void**>(&d->attn_part),
                           sizeof(float) * static_cast<size_t>(c.n_heads) * d->max_splits * kPartStride);
@@ -522,7 +583,7 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
         if (e == hipSuccess)
             e = hipMemsetAsync(d->counters, 0, sizeof(unsigned) * c.n_heads, ctx().stream);
         if (e == hipSuccess)
-            e = hipMemsetAsync(d->state, 0, 4 * sizeof(int), ctx().stream);
+            e = hipMemsetAsync(d->state, 0, kStateBytes, ctx().stream);
         if (e == hipSuccess)
             e = hipStreamSynchronize(ctx().stream);
         if (e != hipSuccess) {

@@ -66,6 +66,7 @@ struct Int4Args {
     // QKV_ROPE
     int kv_dim;
     float theta;
+    const float* rope_table; // (cos, sin) of the step's position for i < 64, or null: computed here from theta
 };
 
 constexpr int kAuxStream = 2; // "nt": weights are touched once
@@ -223,11 +224,16 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     if (item < nitems)
         load_item(cur, cur_res, item);
 
-    if (MODE == QKV_ROPE && threadIdx.x < kRopeHeadSize / 2) {
-        float c, s;
-        rope_cos_sin(c, s, threadIdx.x, kRopeHeadSize, pos, a.theta);
-        rope_tab[2 * threadIdx.x] = c;
-        rope_tab[2 * threadIdx.x + 1] = s;
+    if (MODE == QKV_ROPE) {
+        if (a.rope_table) { // prepared by the kernel that set the position
+            if (threadIdx.x < kRopeHeadSize)
+                rope_tab[threadIdx.x] = a.rope_table[threadIdx.x];
+        } else if (threadIdx.x < kRopeHeadSize / 2) {
+            float c, s;
+            rope_cos_sin(c, s, threadIdx.x, kRopeHeadSize, pos, a.theta);
+            rope_tab[2 * threadIdx.x] = c;
+            rope_tab[2 * threadIdx.x + 1] = s;
+        }
     }
     if (STAGE == STAGE_RMSNORM) {
         if (a.embedding && blockIdx.x == 0) { // the residual stream starts as the embedding row
