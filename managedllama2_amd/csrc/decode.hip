@@ -22,14 +22,26 @@
 namespace l2 {
 
 // ---------------------------------------------------------------- fused attention
-// One workgroup per (head, block of 128 timesteps).  Every byte of K and V the
-// workgroup needs is requested before the first score is computed (16 loads of
-// 16 bytes per lane), 16 lanes share one timestep, scores are rounded to fp16
-// like the reference's `attention` buffer, softmax statistics are per block and
-// the blocks of a head are merged by whichever workgroup finishes last
-// (fixed merge order: deterministic).
-constexpr int kSplitT = 128;
+// One workgroup of 16 wavefronts per (head, block of timesteps).  Every byte of K
+// and V the workgroup needs is requested before the first score is computed (up
+// to 16 loads of 16 bytes per lane; rows outside the block are out of the
+// buffer's range and cost no traffic), 16 lanes share one timestep, scores are
+// rounded to fp16 like the reference's `attention` buffer, softmax statistics
+// are per block and the blocks of a head are merged by whichever workgroup
+// finishes last (fixed merge order: deterministic).
+//
+// One compute unit pulls only a few tens of GB/s, the exchange between
+// workgroups costs about 3 us (write-through stores, an atomic, two dependent
+// reads) and dispatching many 1024-thread workgroups that find nothing to do is
+// not free either (blocks of 128 or 256 rows measured slower at every length).
+// So a block is 512 rows: up to that length a head is one workgroup and needs
+// no exchange at all.
+constexpr int kAttnWaves = 16;
+constexpr int kSplitT = 32 * kAttnWaves; // 512
+constexpr int kMaxSplits = 64; // one lane per block in the merge
 constexpr int kPartStride = kRopeHeadSize + 2; // 128 partial outputs, block max, block sum
+
+inline int attn_max_splits(int seq_len) { return ceil_div(seq_len, kSplitT); }
 
 struct AttnArgs {
     const uint16_t* q;
@@ -45,38 +57,37 @@ struct AttnArgs {
     float scale;
 };
 
-__global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
 {
-    __shared__ float sc[kSplitT];
-    __shared__ float red[16][kRopeHeadSize];
+    constexpr int GROUPS = WAVES * 4;   // 16-lane groups, one timestep each per pass
+    constexpr int SPLIT_T = GROUPS * 8; // timesteps per workgroup
+    __shared__ float sc[SPLIT_T];
+    __shared__ float red[WAVES][kRopeHeadSize];
     __shared__ int is_last;
     const int split = blockIdx.x, h = blockIdx.y;
     const int S = a.pos_ptr ? a.pos_ptr[0] + 1 : a.seq; // attends rows 0..pos (src/Transformer.cs:175)
-    const int nsplit = (S + kSplitT - 1) / kSplitT;
+    const int nsplit = (S + SPLIT_T - 1) / SPLIT_T;
     if (split >= nsplit)
         return;
-    const int t0 = split * kSplitT;
-    const int t1 = S < t0 + kSplitT ? S : t0 + kSplitT;
+    const int t0 = split * SPLIT_T;
+    const int t1 = S < t0 + SPLIT_T ? S : t0 + SPLIT_T;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int l16 = lane & 15, grp = wave * 4 + (lane >> 4);
-    const size_t col = static_cast<size_t>(h) * kRopeHeadSize + l16 * 8;
+    const int col = h * kRopeHeadSize + l16 * 8;
 
+    const uint32_t cache_bytes = static_cast<uint32_t>(t1) * a.dim * 2; // rows of this block only; < 2^31: checked on the host
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(a.kcache, cache_bytes), rv = make_rsrc(a.vcache, cache_bytes);
     const u32x4 qv = *reinterpret_cast<const u32x4*>(a.q + col);
     u32x4 kv[8], vv[8];
-    bool ok[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int t = t0 + i * 16 + grp;
-        ok[i] = t < t1;
-        const size_t off = static_cast<size_t>(ok[i] ? t : t0) * a.dim + col;
-        kv[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.kcache + off));
-    }
+    for (int i = 0; i < 8; ++i)
+        kv[i] = __builtin_amdgcn_raw_buffer_load_b128(rk, ((t0 + i * GROUPS + grp) * a.dim + col) * 2, 0,
+                                                      kAuxNonTemporal);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int t = t0 + i * 16 + grp;
-        const size_t off = static_cast<size_t>(ok[i] ? t : t0) * a.dim + col;
-        vv[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(a.vcache + off));
-    }
+    for (int i = 0; i < 8; ++i)
+        vv[i] = __builtin_amdgcn_raw_buffer_load_b128(rv, ((t0 + i * GROUPS + grp) * a.dim + col) * 2, 0,
+                                                      kAuxNonTemporal);
     float s[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -85,13 +96,21 @@ __global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
         for (int k = 0; k < 4; ++k)
             acc = dot2(kv[i][k], qv[k], acc);
         acc = row16_sum(acc) * a.scale; // native/mat_vec_kernel.cu:71-74
-        s[i] = ok[i] ? half_bits_to_float(float_to_half_bits(acc)) : -INFINITY;
+        s[i] = t0 + i * GROUPS + grp < t1 ? half_bits_to_float(float_to_half_bits(acc)) : -INFINITY;
         if (l16 == 0)
-            sc[i * 16 + grp] = s[i];
+            sc[i * GROUPS + grp] = s[i];
     }
     __syncthreads();
-    const float m = wave_max(fmaxf(sc[lane], sc[lane + 64]));
-    const float l = wave_sum(expf(sc[lane] - m) + expf(sc[lane + 64] - m));
+    float m = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < SPLIT_T / 64; ++k)
+        m = fmaxf(m, sc[lane + 64 * k]);
+    m = wave_max(m);
+    float l = 0.0f;
+#pragma unroll
+    for (int k = 0; k < SPLIT_T / 64; ++k)
+        l += expf(sc[lane + 64 * k] - m);
+    l = wave_sum(l);
     float o[8];
 #pragma unroll
     for (int k = 0; k < 8; ++k)
@@ -107,13 +126,20 @@ __global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
         }
     }
 #pragma unroll
-    for (int k = 0; k < 8; ++k)
-        red[grp][l16 * 8 + k] = o[k];
+    for (int k = 0; k < 8; ++k) { // the 4 groups of a wavefront, then the wavefronts through LDS
+        o[k] += __shfl_xor(o[k], 16, 64);
+        o[k] += __shfl_xor(o[k], 32, 64);
+    }
+    if (lane < 16) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            red[wave][l16 * 8 + k] = o[k];
+    }
     __syncthreads();
     float val = 0.0f;
     if (threadIdx.x < kRopeHeadSize) {
 #pragma unroll
-        for (int g = 0; g < 16; ++g)
+        for (int g = 0; g < WAVES; ++g)
             val += red[g][threadIdx.x];
     }
     uint16_t* out = a.out + static_cast<size_t>(h) * kRopeHeadSize;
@@ -140,12 +166,20 @@ __global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
         store_agent(&a.counters[h], 0u); // ready for the next launch
     // Merge the blocks of this head.  The partials are read with agent-scope
     // buffer loads (they were written by other workgroups of this launch); a read
-    // beyond the last block returns 0, so the loads are unconditional and many of
-    // them are in flight at once.
+    // beyond the last block returns 0, so the loads are unconditional, and the
+    // first eight blocks' outputs are requested before the weights are known.
     const __amdgpu_buffer_rsrc_t rp = make_rsrc(a.part + static_cast<size_t>(h) * a.max_splits * kPartStride,
                                                 static_cast<uint32_t>(nsplit) * kPartStride * sizeof(float));
-    float* wsh = sc;       // per-block weights exp(m_i - M)   (nsplit <= 64 <= kSplitT)
+    float* wsh = sc;         // per-block weights exp(m_i - M)   (nsplit <= kMaxSplits <= SPLIT_T)
     float* lsh = &red[0][0]; // the merged denominator
+    const int j = threadIdx.x & (kRopeHeadSize - 1);
+    float v[8] = {};
+    if (threadIdx.x < kRopeHeadSize) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            v[u] = __builtin_bit_cast(float,
+                                      __builtin_amdgcn_raw_buffer_load_b32(rp, (u * kPartStride + j) * 4, 0, kAuxAgent));
+    }
     if (threadIdx.x < 64) { // one wavefront: block i in lane i
         const int off = (threadIdx.x * kPartStride + kRopeHeadSize) * 4;
         const bool have = static_cast<int>(threadIdx.x) < nsplit;
@@ -161,16 +195,17 @@ __global__ __launch_bounds__(256) void fused_attn_kernel(AttnArgs a)
     __syncthreads();
     if (threadIdx.x < kRopeHeadSize) {
         float O = 0.0f;
-        for (int i0 = 0; i0 < nsplit; i0 += 8) { // block order is fixed: deterministic
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                v[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                                                     rp, ((i0 + u) * kPartStride + static_cast<int>(threadIdx.x)) * 4, 0,
-                                                     kAuxAgent));
+        for (int i0 = 0;;) { // block order is fixed: deterministic
 #pragma unroll
             for (int u = 0; u < 8; ++u)
                 O = fmaf(i0 + u < nsplit ? wsh[i0 + u] : 0.0f, v[u], O);
+            i0 += 8;
+            if (i0 >= nsplit)
+                break;
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                v[u] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                     rp, ((i0 + u) * kPartStride + j) * 4, 0, kAuxAgent));
         }
         out[threadIdx.x] = float_to_half_bits(O / lsh[0]);
     }
@@ -388,7 +423,8 @@ int forward_fused(llama2_decoder* d)
             a.part = d->attn_part, a.counters = d->counters, a.pos_ptr = d->state;
             a.dim = dim, a.max_splits = d->max_splits;
             a.scale = 1.0f / sqrtf(static_cast<float>(d->head_size));
-            hipLaunchKernelGGL(fused_attn_kernel, dim3(d->max_splits, c.n_heads), dim3(256), 0, ctx().stream, a);
+            hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(d->max_splits, c.n_heads), dim3(kAttnWaves * 64), 0,
+                               ctx().stream, a);
             L2_LAUNCH_CHECK("fused attention");
         }
         {
@@ -491,14 +527,17 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
              n_heads);
     L2_CHECK(aligned(query, 16) && aligned(key, 16) && aligned(value, 16), "%s: q/k/v must be 16-byte aligned", fn);
     L2_CHECK(n_heads <= kMaxAttnHeads, "%s: n_heads=%d exceeds %d", fn, n_heads, kMaxAttnHeads);
-    const int splits = ceil_div(seq_length, kSplitT);
+    L2_CHECK((static_cast<long long>(seq_length) + kSplitT) * dim * 2 < (1ll << 31),
+             "%s: seq_length * dim = %lld is too large", fn, static_cast<long long>(seq_length) * dim);
+    const int splits = attn_max_splits(seq_length);
+    L2_CHECK(splits <= kMaxSplits, "%s: seq_length=%d exceeds %d", fn, seq_length, kMaxSplits * kSplitT);
     if (splits > 1)
         L2_TRY(ensure_attn_partials(sizeof(float) * static_cast<size_t>(n_heads) * splits * kPartStride));
     AttnArgs a{};
     a.q = query, a.kcache = key, a.vcache = value, a.out = output;
     a.part = ctx().attn_partials, a.counters = ctx().attn_counters, a.pos_ptr = nullptr, a.seq = seq_length;
     a.dim = dim, a.max_splits = splits, a.scale = scale;
-    hipLaunchKernelGGL(fused_attn_kernel, dim3(splits, n_heads), dim3(256), 0, ctx().stream, a);
+    hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(splits, n_heads), dim3(kAttnWaves * 64), 0, ctx().stream, a);
     L2_LAUNCH_CHECK(fn);
     return LLAMA2_OK;
 }
@@ -539,6 +578,10 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
                         "%s: the fused step needs head_size 128 and dim, hidden_dim multiples of 8 up to 16384 "
                         "(got head_size %d, dim %d, hidden_dim %d); use LLAMA2_DECODE_MODULES",
                         fn, head_size, c.dim, c.hidden_dim);
+        if (attn_max_splits(c.seq_len) > kMaxSplits ||
+            (static_cast<long long>(c.seq_len) + kSplitT) * c.dim * 2 >= (1ll << 31))
+            return fail(LLAMA2_ERR_UNSUPPORTED, "%s: seq_len=%d is too long for the fused attention (dim %d)", fn,
+                        c.seq_len, c.dim);
     }
     L2_CHECK(weights->token_embedding_table && weights->classifier_weights && weights->rms_final_weight &&
                  weights->layers,
@@ -573,7 +616,7 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     d->kv_dim = kv_dim;
     d->head_size = c.dim / c.n_heads;
     if (fused) {
-        d->max_splits = ceil_div(c.seq_len, kSplitT);
+        d->max_splits = attn_max_splits(c.seq_len);
         hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->state), kStateBytes);
         if (e == hipSuccess)
             e = hipMalloc(reinterpret_cast<void**>(&d->attn_part),

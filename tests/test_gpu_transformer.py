@@ -92,7 +92,7 @@ def test_fused_step_tracks_module_step(oracle):
     well below the oracle tolerance."""
     model = synth.random_model(HS128, seed=8, rms_random=True)
     rng = synth.rng_for(405)
-    prompt = rng.integers(3, HS128["vocab_size"], 150).astype(np.int32)  # forces 2 attention blocks
+    prompt = rng.integers(3, HS128["vocab_size"], 150).astype(np.int32)
     outs = []
     for mode in (capi.DECODE_MODULES, FUSED, FUSED_GRAPH):
         t = Transformer(dict(HS128), model, mode=mode)
@@ -104,6 +104,38 @@ def test_fused_step_tracks_module_step(oracle):
     assert np.array_equal(outs[1][0], outs[2][0])  # graph replay == eager launches, bit for bit
     assert_close_normwise(outs[1][0], outs[0][0], "fused vs modules logits", 2e-3)
     assert_close_normwise(outs[1][1].astype(np.float64), outs[0][1].astype(np.float64), "fused vs modules K cache", 2e-3)
+
+
+@pytest.mark.parametrize("pos", [511, 512, 1100])
+def test_fused_step_with_long_history(oracle, pos):
+    """A step whose history spans one, two and three 512-row attention blocks:
+    the caches are filled with random rows, then one step of the module
+    sequence, the fused launches, the graph replay and the oracle are compared."""
+    cfg = dict(HS128, seq_len=1200)
+    dim, L, S = cfg["dim"], cfg["n_layers"], cfg["seq_len"]
+    model = synth.random_model(cfg, seed=11, rms_random=True)
+    rng = synth.rng_for(408, pos)
+    kc = synth.normal_f16(rng, L * S * dim)
+    vc = synth.normal_f16(rng, L * S * dim)
+    token = np.array([17], np.int32)
+    hm = oracle.HostModel(cfg, model)
+    hm.key_cache[:], hm.value_cache[:] = kc, vc
+    hm.tokens[pos] = token[0]
+    want = hm.forward(pos, pos + 1).astype(np.float64)
+    outs = []
+    for mode in (capi.DECODE_MODULES, FUSED, FUSED_GRAPH):
+        t = Transformer(dict(cfg), model, mode=mode)
+        t.runstate.keyCache.copy_to_device(kc)
+        t.runstate.valueCache.copy_to_device(vc)
+        t.runstate.tokens.copy_to_device(token, pos)
+        t.Forward(pos, pos + 1)
+        outs.append(t.runstate.logits.to_host())
+        assert_close_normwise(outs[-1], want, "logits at pos %d, mode %d" % (pos, mode), LOGIT_TOL)
+        row = t.runstate.keyCache.to_host(dim, (L - 1) * S * dim + pos * dim).astype(np.float64)
+        assert_close_normwise(row, hm.key_cache.reshape(L, S, dim)[L - 1, pos].astype(np.float64), "k row", LOGIT_TOL)
+        t.close()
+    assert np.array_equal(outs[1].view(np.uint16), outs[2].view(np.uint16))
+    assert_close_normwise(outs[1], outs[0].astype(np.float64), "fused vs modules", 2e-3)
 
 
 def test_graph_replays_are_stable(oracle):
