@@ -43,6 +43,15 @@
  *   rope .................. identity at pos 0, norm preservation, known angle
  *                           (pos*freq = pi/2 swaps a pair)
  *   argmax ................ numpy.argmax (first maximum)
+ *   softmax_logits ........ two-point closed form, temperature scaling law
+ *                           softmax(x/T), rows sum to 1, indices = 0..n-1
+ *   sort .................. numpy stable argsort of the negated keys, python
+ *                           sorted() on small inputs, permutation check
+ *   cumulative_sum ........ numpy integer cumsum (exact regime of
+ *                           test/CumulativeSumTests.cs:51-57), fp64 cumsum
+ *   sample_top_p .......... brute force over all thresholds on small inputs
+ *   sample ................ composition, checked against the empirical
+ *                           distribution for a 4-token vocabulary
  *   forward ............... composition checked module by module
  * Parity unpinned: the fp32 summation ORDER of the reference's CUB
  * warp/block reductions (it only matters below fp16 rounding and the
@@ -513,6 +522,128 @@ ORACLE_API void ref_embedding(uint16_t* x, const uint16_t* table, int dim, const
 }
 
 /* ================================================================== */
+/* Stochastic sampler: src/Sampler.cs:48-67 and its four kernels.        */
+/* ================================================================== */
+
+/* SoftmaxLogits, in place: test/SoftmaxLogitsTests.cs:33-73; the same    */
+/* three roundings to fp16 as native/softmax_logits_kernel.cu:12-53       */
+/* (after the temperature division, after expf, after the normalisation); */
+/* the sum runs over the unrounded exponentials.                          */
+ORACLE_API void ref_softmax_logits(uint16_t* logits, int size, float temperature, int* indices)
+{
+    for (int i = 0; i < size; ++i) {
+        indices[i] = i;
+        float val = h2f(logits[i]);
+        val /= temperature;
+        logits[i] = f2h(val);
+    }
+    float max_val = h2f(logits[0]);
+    for (int i = 1; i < size; ++i)
+        if (h2f(logits[i]) > max_val)
+            max_val = h2f(logits[i]);
+    float sum = 0.0f;
+    for (int i = 0; i < size; ++i) {
+        float v = expf(h2f(logits[i]) - max_val);
+        logits[i] = f2h(v);
+        sum += v;
+    }
+    for (int i = 0; i < size; ++i)
+        logits[i] = f2h(h2f(logits[i]) / sum);
+}
+
+/* Sort, descending by key, values carried along: test/SortTests.cs:38-43 */
+/* (Array.Sort with a descending comparer).  The kernel is a radix sort   */
+/* (native/sort_kernel.cu:28, cub::BlockRadixSort::SortDescending), which */
+/* is STABLE; .NET's Array.Sort is not, which is why the reference's test */
+/* leaves the indices unchecked (test/SortTests.cs:88-89).  This is the   */
+/* stable sort: equal keys keep their input order.  Keys are ordered by   */
+/* the radix sort's total order on fp16 bit patterns (+0 before -0, NaNs  */
+/* at the two ends), which is the numeric order for everything else.      */
+static inline uint32_t sort_rank(uint16_t k) /* larger rank = sorts first */
+{
+    return (k & 0x8000u) ? (uint32_t)(uint16_t)~k : (uint32_t)(k | 0x8000u);
+}
+
+ORACLE_API void ref_sort(uint16_t* keys, int* values, int size)
+{
+    size_t* start = (size_t*)calloc(65537, sizeof(size_t));
+    uint16_t* k2 = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)size);
+    int* v2 = (int*)malloc(sizeof(int) * (size_t)size);
+    for (int i = 0; i < size; ++i)
+        start[65535 - sort_rank(keys[i]) + 1]++; /* bucket 0 = largest key */
+    for (int b = 0; b < 65536; ++b)
+        start[b + 1] += start[b];
+    for (int i = 0; i < size; ++i) {
+        size_t at = start[65535 - sort_rank(keys[i])]++;
+        k2[at] = keys[i];
+        v2[at] = values[i];
+    }
+    memcpy(keys, k2, sizeof(uint16_t) * (size_t)size);
+    memcpy(values, v2, sizeof(int) * (size_t)size);
+    free(start);
+    free(k2);
+    free(v2);
+}
+
+/* CumulativeSum, in place: test/CumulativeSumTests.cs:37-49 (fp32 running */
+/* sum, every prefix rounded to fp16).                                    */
+ORACLE_API void ref_cumulative_sum(uint16_t* values, int size)
+{
+    float cdf = 0.0f;
+    for (int i = 0; i < size; ++i) {
+        cdf += h2f(values[i]);
+        values[i] = f2h(cdf);
+    }
+}
+
+/* SampleTopP: test/SampleTopPTests.cs:34-46 (first index whose value     */
+/* reaches the threshold, the last index if none does).                   */
+ORACLE_API int ref_sample_top_p(const uint16_t* logits, const int* indices, int size, float threshold)
+{
+    int min_index = size - 1;
+    for (int i = 0; i < size; ++i)
+        if (h2f(logits[i]) >= threshold && i < min_index)
+            min_index = i;
+    return indices[min_index];
+}
+
+/* Sampler.Sample: src/Sampler.cs:40-70.  `logits` and `indices` are      */
+/* overwritten like runstate.logits / runstate.indices.  Returns the      */
+/* token; generate_token == 0 returns -1 (the prompt token stays).        */
+ORACLE_API int ref_argmax(const uint16_t* logits, int n);
+ORACLE_API int ref_sample(uint16_t* logits, int* indices, int size, float temperature, float top_p,
+                          float coin, int generate_token)
+{
+    if (!generate_token)
+        return -1;
+    if (temperature == 0.0f)
+        return ref_argmax(logits, size);
+    ref_softmax_logits(logits, size, temperature, indices);
+    float threshold;
+    if (top_p <= 0 || top_p >= 1) {
+        threshold = coin;
+    } else {
+        ref_sort(logits, indices, size);
+        threshold = coin * top_p;
+    }
+    ref_cumulative_sum(logits, size);
+    return ref_sample_top_p(logits, indices, size, threshold);
+}
+
+/* The uniform number in [0, 1) a device-resident sampling loop draws for */
+/* position `pos` from `seed` (splitmix64 of seed + pos, top 24 bits).    */
+/* The reference draws from an unseeded System.Random (src/Sampler.cs:24, */
+/* 42), so any uniform stream is as good as its own.                      */
+ORACLE_API float oracle_coin(uint64_t seed, int pos)
+{
+    uint64_t z = seed + 0x9E3779B97F4A7C15ull * (uint64_t)(pos + 1);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+/* ================================================================== */
 /* fp64 closed forms.  Outputs are double (pre-rounding) so a test can  */
 /* apply its own error metric; *_h helpers round once to fp16.          */
 /* ================================================================== */
@@ -607,6 +738,37 @@ ORACLE_API void f64_softmax(double* out, const uint16_t* x, int size, int n_rows
         }
         for (int i = 0; i < size; ++i)
             o[i] /= sum;
+    }
+}
+
+/* SoftmaxLogits with exact exp and sum.  The two fp16 roundings that the */
+/* in-place buffer forces on the INPUT of later steps are kept: the       */
+/* temperature division (fp32, correctly rounded, then fp16) and the fp16 */
+/* exponential that is normalised.  out = double(half(e)) / sum(e).       */
+ORACLE_API void f64_softmax_logits(double* out, const uint16_t* logits, int size, float temperature)
+{
+    double m = -INFINITY;
+    for (int i = 0; i < size; ++i) {
+        out[i] = (double)h2f(f2h(h2f(logits[i]) / temperature));
+        if (out[i] > m)
+            m = out[i];
+    }
+    double sum = 0.0;
+    for (int i = 0; i < size; ++i) {
+        double e = exp(out[i] - m);
+        sum += e;
+        out[i] = (double)h2f(d2h(e));
+    }
+    for (int i = 0; i < size; ++i)
+        out[i] /= sum;
+}
+
+ORACLE_API void f64_cumulative_sum(double* out, const uint16_t* values, int size)
+{
+    double cdf = 0.0;
+    for (int i = 0; i < size; ++i) {
+        cdf += (double)h2f(values[i]);
+        out[i] = cdf;
     }
 }
 

@@ -70,6 +70,10 @@ def lib():
         _lib.oracle_d2h.restype = C.c_uint16
         _lib.oracle_d2h.argtypes = [C.c_double]
         _lib.ref_argmax.restype = C.c_int
+        _lib.ref_sample_top_p.restype = C.c_int
+        _lib.ref_sample.restype = C.c_int
+        _lib.oracle_coin.restype = C.c_float
+        _lib.oracle_coin.argtypes = [C.c_uint64, C.c_int]
     return _lib
 
 
@@ -202,6 +206,63 @@ def ref_embedding(table, dim, tokens, pos):
     tokens = np.ascontiguousarray(tokens, np.int32)
     lib().ref_embedding(_h(x), _h(table), C.c_int(dim), tokens.ctypes.data_as(i32p), C.c_int(pos))
     return x
+
+
+# ---- stochastic sampler (src/Sampler.cs:48-67) ------------------------------------------
+def _i(a):
+    assert a.dtype == np.int32 and a.flags.c_contiguous
+    return a.ctypes.data_as(i32p)
+
+
+def ref_softmax_logits(logits, temperature):
+    """-> (probabilities fp16, indices int32)"""
+    out = np.array(logits, np.float16, copy=True)
+    indices = np.empty(out.size, np.int32)
+    lib().ref_softmax_logits(_h(out), C.c_int(out.size), C.c_float(temperature), _i(indices))
+    return out, indices
+
+
+def ref_sort(keys, values):
+    k = np.array(keys, np.float16, copy=True)
+    v = np.array(values, np.int32, copy=True)
+    lib().ref_sort(_h(k), _i(v), C.c_int(k.size))
+    return k, v
+
+
+def ref_cumulative_sum(values):
+    out = np.array(values, np.float16, copy=True)
+    lib().ref_cumulative_sum(_h(out), C.c_int(out.size))
+    return out
+
+
+def ref_sample_top_p(cdf, indices, threshold):
+    cdf = np.ascontiguousarray(cdf, np.float16)
+    indices = np.ascontiguousarray(indices, np.int32)
+    return int(lib().ref_sample_top_p(_h(cdf), _i(indices), C.c_int(cdf.size), C.c_float(threshold)))
+
+
+def ref_sample(logits, temperature, top_p, coin, generate_token=True):
+    """Sampler.Sample on a copy of the logits -> token (-1 when nothing is generated)."""
+    work = np.array(logits, np.float16, copy=True)
+    indices = np.zeros(work.size, np.int32)
+    return int(lib().ref_sample(_h(work), _i(indices), C.c_int(work.size), C.c_float(temperature),
+                                C.c_float(top_p), C.c_float(coin), C.c_int(1 if generate_token else 0)))
+
+
+def coin(seed, pos):
+    return float(lib().oracle_coin(C.c_uint64(seed), C.c_int(pos)))
+
+
+def f64_softmax_logits(logits, temperature):
+    out = np.empty(logits.size, np.float64)
+    lib().f64_softmax_logits(_d(out), _h(logits), C.c_int(logits.size), C.c_float(temperature))
+    return out
+
+
+def f64_cumulative_sum(values):
+    out = np.empty(values.size, np.float64)
+    lib().f64_cumulative_sum(_d(out), _h(values), C.c_int(values.size))
+    return out
 
 
 # ---- fp64 closed forms ------------------------------------------------------------
