@@ -48,6 +48,9 @@ typedef uint16_t llama2_half;
 
 /* Largest softmax row, as in the reference (native/softmax_kernel.cu:5). */
 #define LLAMA2_MAX_SOFTMAX_SIZE 8192
+/* Largest `size` of the sampler modules (softmax_logits, sort, cumulative_sum,
+ * sample_top_p): one 1024-thread workgroup holds the whole vector. */
+#define LLAMA2_MAX_SAMPLER_SIZE 65536
 
 /* ---------------------------------------------------------------- runtime */
 
@@ -219,6 +222,45 @@ int llama2_argmax(const llama2_half* input, int size, int* result, int pos, int 
 int llama2_embedding(llama2_half* output, const llama2_half* table, int size, const int* tokens,
                      int pos);
 
+/* ------------------------------------------------ stochastic sampler modules
+ * The four kernels of Sampler.Sample's temperature / top-p branch
+ * (src/Sampler.cs:48-67).  1 <= size <= LLAMA2_MAX_SAMPLER_SIZE (the
+ * reference's launch shapes fix size to a multiple of 125 resp. 32 up to
+ * 32000; any size works here).  fp16 and int buffers 16-byte aligned. */
+
+/* softmax_logits_kernel (native/softmax_logits_kernel.cuh:5), module
+ * SoftmaxLogits.Forward (src/SoftmaxLogits.cs:14-15): indices[t] = t;
+ * logits <- softmax(logits / temperature) in place with the reference's three
+ * fp16 roundings (after the division, after expf, after the normalisation).
+ * temperature > 0. */
+int llama2_softmax_logits(llama2_half* logits, int size, float temperature, int* indices);
+
+/* sort_kernel (native/sort_kernel.cuh:4), module Sort.Forward
+ * (src/Sort.cs:14-15): sorts keys in DESCENDING order, in place, carrying
+ * values along.  Stable (equal keys keep their order), like the reference's
+ * cub::BlockRadixSort; keys are ordered as the radix sort orders fp16 bit
+ * patterns (numeric order, +0 before -0, NaNs at the two ends). */
+int llama2_sort(llama2_half* keys, int* values, int size);
+
+/* cumulative_sum_kernel (native/cumulative_sum_kernel.cuh:5), module
+ * CumulativeSum.Forward (src/CumulativeSum.cs:14-15): in-place inclusive
+ * prefix sums, accumulated in fp32, each rounded to fp16. */
+int llama2_cumulative_sum(llama2_half* values, int size);
+
+/* sample_top_p_kernel (native/sample_top_p_kernel.cuh:5), module
+ * SampleTopP.Forward (src/SampleTopP.cs:14-15): result[pos] = indices[m], m the
+ * first position with float(logits[m]) >= threshold, or size-1 if none. */
+int llama2_sample_top_p(const llama2_half* logits, const int* indices, int size, float threshold,
+                        int* result, int pos);
+
+/* The stochastic branch of Sampler.Sample (src/Sampler.cs:50-66) as ONE launch:
+ * softmax_logits; if 0 < top_p < 1: sort and threshold = coin * top_p, else
+ * threshold = coin; cumulative_sum; sample_top_p into result[pos].  logits and
+ * indices are overwritten exactly as by the four module calls (same device
+ * code).  coin is the caller's uniform number in [0, 1). */
+int llama2_sample(llama2_half* logits, int* indices, int size, float temperature, float top_p,
+                  float coin, int* result, int pos);
+
 /* ------------------------------------------------------------ decode step */
 
 /* src/Config.cs:6-19 -- the 32-byte model-file header, same field order. */
@@ -256,7 +298,9 @@ typedef struct llama2_transformer_weights {
 } llama2_transformer_weights;
 
 /* src/RunState.cs:7-25.  attention holds n_heads*max(dim, seq_len) halfs,
- * key/value caches n_layers*seq_len*kv_dim halfs, tokens seq_len+1 ints. */
+ * key/value caches n_layers*seq_len*kv_dim halfs, tokens seq_len+1 ints,
+ * indices vocab_size ints (only the stochastic sampler uses it: may be null
+ * for greedy decoding). */
 typedef struct llama2_run_state {
     llama2_half* x;
     llama2_half* xb;
@@ -267,6 +311,7 @@ typedef struct llama2_run_state {
     llama2_half* key_cache;
     llama2_half* value_cache;
     int* tokens;
+    int* indices;
 } llama2_run_state;
 
 typedef struct llama2_decoder llama2_decoder;
@@ -291,11 +336,27 @@ int llama2_decode_forward(llama2_decoder* decoder, int position, int next_positi
  * (the one host synchronisation per token). */
 int llama2_decode_sample(llama2_decoder* decoder, int next_position, int generate_token,
                          int* token);
+/* Sampler.Sample with temperature and top-p (src/Sampler.cs:40-70): the greedy
+ * branch when temperature == 0 or !generate_token, otherwise llama2_sample on
+ * state->logits / state->indices with the caller's uniform `coin` in [0, 1);
+ * then reads tokens[next_position] back. */
+int llama2_decode_sample_top_p(llama2_decoder* decoder, int next_position, int generate_token,
+                               float temperature, float top_p, float coin, int* token);
+/* The uniform number the device-resident sampling loop draws for the token at
+ * `position` from `seed` (splitmix64 of seed + position, top 24 bits); exported
+ * so that a host loop can reproduce llama2_decode_run_sampled step by step. */
+float llama2_sampler_coin(unsigned long long seed, int position);
 /* `steps` iterations of forward + greedy sample starting at `position`
  * without any host synchronisation in between (tokens stay on the device;
  * positions below n_prompt keep their prompt token, as Transformer.Generate
  * does, src/Transformer.cs:96-104).  Does not stop on token < 3. */
 int llama2_decode_run(llama2_decoder* decoder, int position, int steps, int n_prompt);
+/* The same loop with the stochastic sampler: the token at next_position p is
+ * drawn with coin = llama2_sampler_coin(seed, p).  temperature == 0 is
+ * llama2_decode_run.  (The reference draws from an unseeded System.Random,
+ * src/Sampler.cs:24,42, on the host; this keeps the loop on the device.) */
+int llama2_decode_run_sampled(llama2_decoder* decoder, int position, int steps, int n_prompt,
+                              float temperature, float top_p, unsigned long long seed);
 int llama2_decode_destroy(llama2_decoder* decoder);
 
 #if defined(__GNUC__)

@@ -14,6 +14,7 @@ ERR_NOT_INITIALIZED = -2
 ERR_UNSUPPORTED = -3
 ERR_NO_DEVICE = -4
 MAX_SOFTMAX_SIZE = 8192
+MAX_SAMPLER_SIZE = 65536
 
 DECODE_MODULES = 0
 DECODE_FUSED = 1
@@ -61,7 +62,7 @@ class TransformerWeights(C.Structure):
 class RunState(C.Structure):
     """src/RunState.cs:7-25"""
     _fields_ = [("x", vp), ("xb", vp), ("h", vp), ("q", vp), ("attention", vp), ("logits", vp),
-                ("key_cache", vp), ("value_cache", vp), ("tokens", vp)]
+                ("key_cache", vp), ("value_cache", vp), ("tokens", vp), ("indices", vp)]
 
 
 _SIGNATURES = {
@@ -96,15 +97,23 @@ _SIGNATURES = {
     "llama2_softmax": [vp, i, i],
     "llama2_argmax": [vp, i, vp, i, i],
     "llama2_embedding": [vp, vp, i, vp, i],
+    "llama2_softmax_logits": [vp, i, f, vp],
+    "llama2_sort": [vp, vp, i],
+    "llama2_cumulative_sum": [vp, i],
+    "llama2_sample_top_p": [vp, vp, i, f, vp, i],
+    "llama2_sample": [vp, vp, i, f, f, f, vp, i],
     "llama2_decode_create": [C.POINTER(vp), C.POINTER(Config), C.POINTER(TransformerWeights),
                              C.POINTER(RunState), i],
     "llama2_decode_forward": [vp, i, i],
     "llama2_decode_sample": [vp, i, i, C.POINTER(i)],
+    "llama2_decode_sample_top_p": [vp, i, i, f, f, f, C.POINTER(i)],
     "llama2_decode_run": [vp, i, i, i],
+    "llama2_decode_run_sampled": [vp, i, i, i, f, f, C.c_ulonglong],
     "llama2_decode_destroy": [vp],
 }
 # exported, not status-returning
-_OTHER = {"llama2_last_error": (C.c_char_p, []), "llama2_stream": (vp, [])}
+_OTHER = {"llama2_last_error": (C.c_char_p, []), "llama2_stream": (vp, []),
+          "llama2_sampler_coin": (f, [C.c_ulonglong, i])}
 
 EXPORTS = sorted(list(_SIGNATURES) + list(_OTHER))
 

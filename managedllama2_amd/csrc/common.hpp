@@ -24,6 +24,9 @@ struct Context {
     size_t attn_partials_bytes = 0;
     // per-head arrival counters of llama2_multi_head_attention (zero between launches)
     unsigned* attn_counters = nullptr;
+    // second buffer of the sampler's radix sort (LLAMA2_MAX_SAMPLER_SIZE keys and payloads)
+    uint16_t* sort_keys = nullptr;
+    int* sort_values = nullptr;
 };
 
 constexpr int kMaxAttnHeads = 1024;

@@ -13,6 +13,7 @@
 //                          is identical for every token and can be replayed as
 //                          one hipGraph (LLAMA2_DECODE_GRAPH).
 #include "int4_kernels.hpp"
+#include "sampler_kernels.hpp"
 
 #include <climits>
 #include <cmath>
@@ -312,6 +313,30 @@ __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, in
     }
 }
 
+// Sampler.Sample's stochastic branch (src/Sampler.cs:48-67) against the device
+// state: the token at pos+1 is drawn with the coin of (seed, pos+1) iff
+// pos+1 >= n_prompt; then the position advances like in argmax_step_kernel.
+template <int CH>
+__global__ __launch_bounds__(kSampBlock) void sample_step_kernel(uint16_t* logits, int* indices, int size, int* tokens,
+                                                                 int* state, uint16_t* keys2, int* values2,
+                                                                 float temperature, float top_p,
+                                                                 unsigned long long seed, float theta)
+{
+    __shared__ SamplerLds lds;
+    const int pos0 = state[0], n_prompt = state[1], advance0 = state[2];
+    if (advance0 && threadIdx.x >= 64 && threadIdx.x < 64 + kRopeHeadSize / 2)
+        write_rope_table(state, threadIdx.x - 64, pos0 + 1, theta); // for the next step
+    if (pos0 + 1 >= n_prompt) { // uniform over the workgroup
+        const int token = sample_dev<CH>(logits, indices, size, temperature, top_p, sampler_coin(seed, pos0 + 1),
+                                         keys2, values2, lds);
+        if (threadIdx.x == 0)
+            tokens[pos0 + 1] = token;
+    }
+    __syncthreads(); // every thread has read the state
+    if (threadIdx.x == 0 && advance0)
+        state[0] = pos0 + 1;
+}
+
 } // namespace l2
 
 struct llama2_decoder {
@@ -329,6 +354,10 @@ struct llama2_decoder {
     int max_splits = 0;
     hipGraphExec_t graph_forward = nullptr; // Transformer.Forward
     hipGraphExec_t graph_step = nullptr;    // Forward + greedy sample + position advance
+    // Forward + stochastic sample + position advance, captured for the parameters below
+    hipGraphExec_t graph_step_sampled = nullptr;
+    float sampled_temperature = 0.0f, sampled_top_p = 0.0f;
+    unsigned long long sampled_seed = 0;
 };
 
 using namespace l2;
@@ -460,6 +489,32 @@ int launch_argmax_step(llama2_decoder* d)
     return LLAMA2_OK;
 }
 
+int launch_sample_step(llama2_decoder* d, float temperature, float top_p, unsigned long long seed)
+{
+    const int size = d->cfg.vocab_size;
+    if (size <= 4 * 8 * kSampBlock)
+        hipLaunchKernelGGL(sample_step_kernel<4>, dim3(1), dim3(kSampBlock), 0, ctx().stream, d->s.logits, d->s.indices,
+                           size, d->s.tokens, d->state, ctx().sort_keys, ctx().sort_values, temperature, top_p, seed,
+                           d->cfg.rope_theta);
+    else
+        hipLaunchKernelGGL(sample_step_kernel<8>, dim3(1), dim3(kSampBlock), 0, ctx().stream, d->s.logits, d->s.indices,
+                           size, d->s.tokens, d->state, ctx().sort_keys, ctx().sort_values, temperature, top_p, seed,
+                           d->cfg.rope_theta);
+    L2_LAUNCH_CHECK("sample_step_kernel");
+    return LLAMA2_OK;
+}
+
+int check_sampling(const char* fn, const llama2_decoder* d, float temperature)
+{
+    L2_CHECK(temperature > 0.0f, "%s: temperature=%g must be positive", fn, static_cast<double>(temperature));
+    L2_CHECK(d->s.indices, "%s: the run state has no indices buffer (vocab_size ints)", fn);
+    L2_CHECK(aligned(d->s.indices, 16), "%s: run-state indices must be 16-byte aligned", fn);
+    if (d->cfg.vocab_size > LLAMA2_MAX_SAMPLER_SIZE)
+        return fail(LLAMA2_ERR_UNSUPPORTED, "%s: vocab_size=%d exceeds the sampler limit %d", fn, d->cfg.vocab_size,
+                    LLAMA2_MAX_SAMPLER_SIZE);
+    return LLAMA2_OK;
+}
+
 int set_state(llama2_decoder* d, int pos, int n_prompt, int advance)
 {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, ctx().stream, d->state, pos, n_prompt, advance,
@@ -468,13 +523,14 @@ int set_state(llama2_decoder* d, int pos, int n_prompt, int advance)
     return LLAMA2_OK;
 }
 
-int capture(hipGraphExec_t* exec, llama2_decoder* d, bool with_sample)
+int capture(hipGraphExec_t* exec, llama2_decoder* d, bool with_sample, bool stochastic = false)
 {
     L2_HIP(hipStreamBeginCapture(ctx().stream, hipStreamCaptureModeThreadLocal));
     ctx().capturing = true;
     int rc = forward_fused(d);
     if (rc == LLAMA2_OK && with_sample)
-        rc = launch_argmax_step(d);
+        rc = stochastic ? launch_sample_step(d, d->sampled_temperature, d->sampled_top_p, d->sampled_seed)
+                        : launch_argmax_step(d);
     ctx().capturing = false;
     hipGraph_t g = nullptr;
     hipError_t e = hipStreamEndCapture(ctx().stream, &g);
@@ -498,6 +554,8 @@ void release(llama2_decoder* d)
         (void)hipGraphExecDestroy(d->graph_forward);
     if (d->graph_step)
         (void)hipGraphExecDestroy(d->graph_step);
+    if (d->graph_step_sampled)
+        (void)hipGraphExecDestroy(d->graph_step_sampled);
     if (d->state)
         (void)hipFree(d->state);
     if (d->attn_part)
@@ -673,6 +731,67 @@ int llama2_decode_sample(llama2_decoder* d, int next_position, int generate_toke
              next_position);
     L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, d->s.tokens, next_position, generate_token));
     return llama2_memcpy_d2h(token, d->s.tokens, static_cast<size_t>(next_position) * sizeof(int), sizeof(int));
+}
+
+int llama2_decode_sample_top_p(llama2_decoder* d, int next_position, int generate_token, float temperature,
+                               float top_p, float coin, int* token)
+{
+    L2_REQUIRE_INIT();
+    const char* fn = "llama2_decode_sample_top_p";
+    L2_CHECK(d && token, "%s: null argument", fn);
+    if (temperature == 0.0f || !generate_token) // src/Sampler.cs:44-47
+        return llama2_decode_sample(d, next_position, generate_token, token);
+    L2_CHECK(next_position >= 0 && next_position <= d->cfg.seq_len, "%s: next_position=%d", fn, next_position);
+    L2_TRY(check_sampling(fn, d, temperature));
+    L2_TRY(llama2_sample(d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p, coin, d->s.tokens,
+                         next_position)); // :50-66
+    return llama2_memcpy_d2h(token, d->s.tokens, static_cast<size_t>(next_position) * sizeof(int), sizeof(int)); // :69
+}
+
+float llama2_sampler_coin(unsigned long long seed, int position) { return sampler_coin(seed, position); }
+
+int llama2_decode_run_sampled(llama2_decoder* d, int position, int steps, int n_prompt, float temperature,
+                              float top_p, unsigned long long seed)
+{
+    L2_REQUIRE_INIT();
+    const char* fn = "llama2_decode_run_sampled";
+    L2_CHECK(d, "%s: null decoder", fn);
+    if (temperature == 0.0f)
+        return llama2_decode_run(d, position, steps, n_prompt);
+    L2_CHECK(position >= 0 && steps >= 0 && position + steps <= d->cfg.seq_len,
+             "%s: position=%d steps=%d exceed seq_len=%d", fn, position, steps, d->cfg.seq_len);
+    L2_TRY(check_sampling(fn, d, temperature));
+    if (!(d->mode & LLAMA2_DECODE_FUSED)) {
+        for (int pos = position; pos < position + steps; ++pos) {
+            L2_TRY(forward_modules(d, pos, pos + 1));
+            if (pos + 1 >= n_prompt)
+                L2_TRY(llama2_sample(d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p,
+                                     sampler_coin(seed, pos + 1), d->s.tokens, pos + 1));
+        }
+        return LLAMA2_OK;
+    }
+    if ((d->mode & LLAMA2_DECODE_GRAPH) && !ctx().capturing &&
+        (!d->graph_step_sampled || d->sampled_temperature != temperature || d->sampled_top_p != top_p ||
+         d->sampled_seed != seed)) {
+        // the sampling parameters are kernel arguments of the captured step: capture again when they change
+        if (d->graph_step_sampled) {
+            L2_HIP(hipStreamSynchronize(ctx().stream));
+            (void)hipGraphExecDestroy(d->graph_step_sampled);
+            d->graph_step_sampled = nullptr;
+        }
+        d->sampled_temperature = temperature, d->sampled_top_p = top_p, d->sampled_seed = seed;
+        L2_TRY(capture(&d->graph_step_sampled, d, true, true));
+    }
+    L2_TRY(set_state(d, position, n_prompt, 1));
+    for (int i = 0; i < steps; ++i) {
+        if (d->graph_step_sampled && !ctx().capturing) {
+            L2_HIP(hipGraphLaunch(d->graph_step_sampled, ctx().stream));
+        } else {
+            L2_TRY(forward_fused(d));
+            L2_TRY(launch_sample_step(d, temperature, top_p, seed));
+        }
+    }
+    return LLAMA2_OK;
 }
 
 int llama2_decode_run(llama2_decoder* d, int position, int steps, int n_prompt)

@@ -79,6 +79,8 @@ int llama2_init(int device)
     L2_HIP(hipStreamCreateWithFlags(&c.stream, hipStreamNonBlocking));
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.attn_counters), kMaxAttnHeads * sizeof(unsigned)));
     L2_HIP(hipMemset(c.attn_counters, 0, kMaxAttnHeads * sizeof(unsigned)));
+    L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_keys), LLAMA2_MAX_SAMPLER_SIZE * sizeof(uint16_t)));
+    L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_values), LLAMA2_MAX_SAMPLER_SIZE * sizeof(int)));
     c.device = device;
     c.ready = true;
     g_err[0] = 0;
@@ -98,6 +100,12 @@ int llama2_shutdown(void)
     if (c.attn_counters)
         L2_HIP(hipFree(c.attn_counters));
     c.attn_counters = nullptr;
+    if (c.sort_keys)
+        L2_HIP(hipFree(c.sort_keys));
+    c.sort_keys = nullptr;
+    if (c.sort_values)
+        L2_HIP(hipFree(c.sort_values));
+    c.sort_values = nullptr;
     L2_HIP(hipStreamDestroy(c.stream));
     c.stream = nullptr;
     c.ready = false;

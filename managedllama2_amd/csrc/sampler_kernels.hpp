@@ -1,0 +1,409 @@
+// The stochastic sampler of src/Sampler.cs:48-67 as device functions for one
+// 1024-thread workgroup: softmax_logits, sort, cumulative_sum, sample_top_p
+// (native/softmax_logits_kernel.cu, sort_kernel.cu, cumulative_sum_kernel.cu,
+// sample_top_p_kernel.cu).  Each module kernel calls one of them; the decode
+// step calls all four from a single launch.
+//
+// 32000 logits are 64 KB: the work is latency-bound, so every phase touches
+// global memory once for reading and once for writing, 16 bytes per access,
+// and keeps its share in registers in between.  CH is the number of 8-element
+// chunks a thread holds: 4 up to 32768 elements, 8 up to 65536.
+#pragma once
+
+#include "common.hpp"
+
+namespace l2 {
+
+constexpr int kSampBlock = 1024;
+constexpr int kSampWaves = kSampBlock / 64;
+
+struct SamplerLds {
+    float redf[kSampWaves];
+    int redi[kSampWaves];
+    uint16_t counts[16 * kSampBlock]; // sort: per (digit, thread) counters, then scatter cursors
+};
+
+// ---- 8-element chunks of fp16 / int32 -----------------------------------------------
+// Whole chunks move as 16-byte accesses, the ragged last chunk element by element.
+__device__ __forceinline__ void load_half8(float (&f)[8], const uint16_t* p, int base, int size, float fill)
+{
+    if (base + 8 <= size) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(p + base);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            f[k] = half_bits_to_float(static_cast<uint16_t>(v[k >> 1] >> (16 * (k & 1))));
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            f[k] = base + k < size ? half_bits_to_float(p[base + k]) : fill;
+    }
+}
+
+__device__ __forceinline__ void load_bits8(uint16_t (&b)[8], const uint16_t* p, int base, int size)
+{
+    if (base + 8 <= size) {
+        const u32x4 v = *reinterpret_cast<const u32x4*>(p + base);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            b[k] = static_cast<uint16_t>(v[k >> 1] >> (16 * (k & 1)));
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            b[k] = base + k < size ? p[base + k] : static_cast<uint16_t>(0);
+    }
+}
+
+__device__ __forceinline__ void store_half8(uint16_t* p, int base, int size, const uint16_t (&b)[8])
+{
+    if (base + 8 <= size) {
+        u32x4 v;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            v[k] = static_cast<uint32_t>(b[2 * k]) | (static_cast<uint32_t>(b[2 * k + 1]) << 16);
+        *reinterpret_cast<u32x4*>(p + base) = v;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (base + k < size)
+                p[base + k] = b[k];
+    }
+}
+
+__device__ __forceinline__ void load_int8(int (&o)[8], const int* p, int base, int size)
+{
+    if (base + 8 <= size) {
+        const u32x4 a = *reinterpret_cast<const u32x4*>(p + base), b = *reinterpret_cast<const u32x4*>(p + base + 4);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            o[k] = static_cast<int>(a[k]);
+            o[4 + k] = static_cast<int>(b[k]);
+        }
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            o[k] = base + k < size ? p[base + k] : 0;
+    }
+}
+
+__device__ __forceinline__ void store_int8(int* p, int base, int size, const int (&o)[8])
+{
+    if (base + 8 <= size) {
+        u32x4 a, b;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            a[k] = static_cast<uint32_t>(o[k]);
+            b[k] = static_cast<uint32_t>(o[4 + k]);
+        }
+        *reinterpret_cast<u32x4*>(p + base) = a;
+        *reinterpret_cast<u32x4*>(p + base + 4) = b;
+    } else {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (base + k < size)
+                p[base + k] = o[k];
+    }
+}
+
+// ---- reductions and scans over the 1024 threads -------------------------------------
+__device__ __forceinline__ float samp_block_sum(float v, float* lds)
+{
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0)
+        lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = (threadIdx.x & 63) < kSampWaves ? lds[threadIdx.x & 63] : 0.0f;
+    t = wave_sum(t);
+    __syncthreads();
+    return t;
+}
+
+__device__ __forceinline__ float samp_block_max(float v, float* lds)
+{
+    v = wave_max(v);
+    if ((threadIdx.x & 63) == 0)
+        lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float t = (threadIdx.x & 63) < kSampWaves ? lds[threadIdx.x & 63] : -INFINITY;
+    t = wave_max(t);
+    __syncthreads();
+    return t;
+}
+
+__device__ __forceinline__ int samp_block_min(int v, int* lds)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const int o = __shfl_xor(v, off, 64);
+        v = o < v ? o : v;
+    }
+    if ((threadIdx.x & 63) == 0)
+        lds[threadIdx.x >> 6] = v;
+    __syncthreads();
+    int t = (threadIdx.x & 63) < kSampWaves ? lds[threadIdx.x & 63] : 0x7FFFFFFF;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const int o = __shfl_xor(t, off, 64);
+        t = o < t ? o : t;
+    }
+    __syncthreads();
+    return t;
+}
+
+// Exclusive prefix of one value per thread, in thread order (fixed association:
+// within a wavefront by doubling, then over the 16 wavefront totals).
+template <typename T>
+__device__ __forceinline__ T samp_block_exclusive_scan(T v, T* lds /* kSampWaves */)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    T inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const T o = __shfl_up(inc, off, 64);
+        if (lane >= off)
+            inc += o;
+    }
+    if (lane == 63)
+        lds[wave] = inc;
+    __syncthreads();
+    T before = 0; // total of the wavefronts in front of this one
+#pragma unroll
+    for (int w = 0; w < kSampWaves; ++w)
+        before += w < wave ? lds[w] : static_cast<T>(0);
+    __syncthreads();
+    return before + inc - v;
+}
+
+// ---- softmax_logits (native/softmax_logits_kernel.cu:8-53) ---------------------------
+// indices[t] = t; logits <- half(logits / temperature); p = expf(l - max) rounded to
+// fp16; logits <- half(float(half(p)) / sum of the unrounded p).  The three fp16
+// roundings are the ones the reference's in-place buffer forces.
+template <int CH>
+__device__ __forceinline__ void softmax_logits_dev(uint16_t* logits, int size, float temperature, int* indices,
+                                                   SamplerLds& lds)
+{
+    float f[CH][8];
+    float m = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int base = (threadIdx.x + c * kSampBlock) * 8;
+        if (base < size) {
+            load_half8(f[c], logits, base, size, -INFINITY);
+            int idx[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                idx[k] = base + k;
+                if (base + k < size) {
+                    f[c][k] = half_bits_to_float(float_to_half_bits(f[c][k] / temperature));
+                    m = fmaxf(m, f[c][k]);
+                }
+            }
+            store_int8(indices, base, size, idx);
+        }
+    }
+    m = samp_block_max(m, lds.redf);
+    float sum = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int base = (threadIdx.x + c * kSampBlock) * 8;
+        if (base < size) {
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                if (base + k < size) {
+                    const float v = expf(f[c][k] - m);
+                    sum += v;
+                    f[c][k] = half_bits_to_float(float_to_half_bits(v));
+                }
+        }
+    }
+    sum = samp_block_sum(sum, lds.redf);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int base = (threadIdx.x + c * kSampBlock) * 8;
+        if (base < size) {
+            uint16_t b[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                b[k] = float_to_half_bits(f[c][k] / sum);
+            store_half8(logits, base, size, b);
+        }
+    }
+}
+
+// ---- sort (native/sort_kernel.cu:13-37) ---------------------------------------------
+// Stable descending radix sort of fp16 keys with int payloads: four passes of
+// four bits over the keys' total order (sign-flipped bit pattern; +0 before -0).
+// Thread t owns the 8*CH consecutive items starting at 8*CH*t, so "thread order,
+// then item order" is the input order and the scatter is stable.  Even passes
+// write (keys2, values2), odd passes write back: the result ends in place.
+__device__ __forceinline__ uint32_t sort_rank(uint16_t k) // larger = sorts first
+{
+    return (k & 0x8000u) ? static_cast<uint32_t>(static_cast<uint16_t>(~k)) : static_cast<uint32_t>(k) | 0x8000u;
+}
+
+template <int CH>
+__device__ __forceinline__ void sort_dev(uint16_t* keys, int* values, int size, uint16_t* keys2, int* values2,
+                                         SamplerLds& lds)
+{
+    const int first = threadIdx.x * 8 * CH;
+    uint16_t* kin = keys;
+    int* vin = values;
+    uint16_t* kout = keys2;
+    int* vout = values2;
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 4 * pass;
+        uint16_t kb[CH][8];
+        uint32_t cnt[4] = {0u, 0u, 0u, 0u}; // 16 byte-wide counters (a thread owns at most 64 items)
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int base = first + c * 8;
+            if (base < size) {
+                load_bits8(kb[c], kin, base, size);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (base + k < size) {
+                        const uint32_t d = 15u - ((sort_rank(kb[c][k]) >> shift) & 15u); // bucket 0 = largest digit
+                        const uint32_t inc = 1u << ((d & 3u) * 8u);
+                        cnt[0] += (d >> 2) == 0u ? inc : 0u;
+                        cnt[1] += (d >> 2) == 1u ? inc : 0u;
+                        cnt[2] += (d >> 2) == 2u ? inc : 0u;
+                        cnt[3] += (d >> 2) == 3u ? inc : 0u;
+                    }
+            }
+        }
+#pragma unroll
+        for (int d = 0; d < 16; ++d)
+            lds.counts[d * kSampBlock + threadIdx.x] = static_cast<uint16_t>((cnt[d >> 2] >> ((d & 3) * 8)) & 0xFFu);
+        __syncthreads();
+        // exclusive scan of the 16 x 1024 counters in (digit, thread) order: 16 consecutive per thread
+        {
+            uint16_t* mine = lds.counts + threadIdx.x * 16;
+            int local[16], total = 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                local[i] = total;
+                total += mine[i];
+            }
+            const int before = samp_block_exclusive_scan<int>(total, lds.redi);
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                mine[i] = static_cast<uint16_t>(before + local[i]); // < 65536: positions of a sort of at most 65536 items
+        }
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int base = first + c * 8;
+            if (base < size) {
+                int vb[8];
+                load_int8(vb, vin, base, size);
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    if (base + k < size) {
+                        const uint32_t d = 15u - ((sort_rank(kb[c][k]) >> shift) & 15u);
+                        uint16_t* cursor = &lds.counts[d * kSampBlock + threadIdx.x]; // only this thread touches it
+                        const int at = *cursor;
+                        *cursor = static_cast<uint16_t>(at + 1);
+                        kout[at] = kb[c][k];
+                        vout[at] = vb[k];
+                    }
+            }
+        }
+        __syncthreads(); // the scattered items are visible to the whole workgroup
+        uint16_t* tk = kin;
+        kin = kout;
+        kout = tk;
+        int* tv = vin;
+        vin = vout;
+        vout = tv;
+    }
+}
+
+// ---- cumulative_sum (native/cumulative_sum_kernel.cu:8-26) ---------------------------
+// Inclusive prefix sums in fp32, each rounded to fp16, in place.  A thread sums
+// its 8*CH consecutive values in order, the thread totals are scanned in thread
+// order, prefix + running sum is stored.
+template <int CH>
+__device__ __forceinline__ void cumulative_sum_dev(uint16_t* values, int size, SamplerLds& lds)
+{
+    const int first = threadIdx.x * 8 * CH;
+    float f[CH][8];
+    float run = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int base = first + c * 8;
+        if (base < size) {
+            load_half8(f[c], values, base, size, 0.0f);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                run += f[c][k];
+                f[c][k] = run;
+            }
+        }
+    }
+    const float before = samp_block_exclusive_scan<float>(run, lds.redf);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int base = first + c * 8;
+        if (base < size) {
+            uint16_t b[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                b[k] = float_to_half_bits(before + f[c][k]);
+            store_half8(values, base, size, b);
+        }
+    }
+}
+
+// ---- sample_top_p (native/sample_top_p_kernel.cu:8-21) -------------------------------
+// The value at the first position whose entry reaches the threshold (the last
+// position if none does) of `indices`; returned in every thread.
+template <int CH>
+__device__ __forceinline__ int sample_top_p_dev(const uint16_t* logits, const int* indices, int size, float threshold,
+                                                SamplerLds& lds)
+{
+    int best = size - 1;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int base = (threadIdx.x + c * kSampBlock) * 8;
+        if (base < size) {
+            float f[8];
+            load_half8(f, logits, base, size, -INFINITY);
+#pragma unroll
+            for (int k = 7; k >= 0; --k)
+                if (base + k < size && f[k] >= threshold && base + k < best)
+                    best = base + k;
+        }
+    }
+    best = samp_block_min(best, lds.redi);
+    return indices[best];
+}
+
+// Uniform number in [0, 1) for position `pos` of the stream `seed`: splitmix64
+// of seed + pos, top 24 bits.  (The reference draws from an unseeded
+// System.Random, src/Sampler.cs:24,42.)
+__host__ __device__ inline float sampler_coin(unsigned long long seed, int pos)
+{
+    unsigned long long z = seed + 0x9E3779B97F4A7C15ull * static_cast<unsigned long long>(pos + 1);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return static_cast<float>(z >> 40) * (1.0f / 16777216.0f);
+}
+
+// Sampler.Sample's stochastic branch (src/Sampler.cs:48-67) on one workgroup.
+template <int CH>
+__device__ __forceinline__ int sample_dev(uint16_t* logits, int* indices, int size, float temperature, float top_p,
+                                          float coin, uint16_t* keys2, int* values2, SamplerLds& lds)
+{
+    softmax_logits_dev<CH>(logits, size, temperature, indices, lds);
+    __syncthreads();
+    float threshold = coin;
+    if (!(top_p <= 0.0f || top_p >= 1.0f)) {
+        sort_dev<CH>(logits, indices, size, keys2, values2, lds);
+        threshold = coin * top_p;
+    }
+    cumulative_sum_dev<CH>(logits, size, lds);
+    __syncthreads();
+    return sample_top_p_dev<CH>(logits, indices, size, threshold, lds);
+}
+
+} // namespace l2

@@ -245,7 +245,7 @@ class TransformerWeights {
 // ---------------------------------------------------------------- src/RunState.cs:5-55
 struct RunState {
     DeviceVariable<Half> x, xb, h, q, attention, logits, keyCache, valueCache;
-    DeviceVariable<int> tokens;
+    DeviceVariable<int> tokens, indices;
 
     RunState(Config& config, int kvDim)
     {
@@ -271,6 +271,7 @@ struct RunState {
         keyCache = DeviceVariable<Half>(kv);
         valueCache = DeviceVariable<Half>(kv);
         tokens = DeviceVariable<int>(config.seq_len + 1);
+        indices = DeviceVariable<int>(config.vocab_size); // :53
         keyCache.Zero();
         valueCache.Zero();
         tokens.Zero();
@@ -278,7 +279,8 @@ struct RunState {
     llama2_run_state View() const
     {
         return {x.DevicePointer(), xb.DevicePointer(), h.DevicePointer(), q.DevicePointer(), attention.DevicePointer(),
-                logits.DevicePointer(), keyCache.DevicePointer(), valueCache.DevicePointer(), tokens.DevicePointer()};
+                logits.DevicePointer(), keyCache.DevicePointer(), valueCache.DevicePointer(), tokens.DevicePointer(),
+                indices.DevicePointer()};
     }
 };
 
@@ -412,20 +414,82 @@ struct Embedding : Module { // src/Embedding.cs
     }
 };
 
-// ---------------------------------------------------------------- src/Sampler.cs (temperature == 0)
+struct SoftmaxLogits : Module { // src/SoftmaxLogits.cs
+    using Module::Module;
+    void Forward(DeviceVariable<Half>& logits, int size, float temperature, DeviceVariable<int>& indices)
+    {
+        Check(llama2_softmax_logits(logits.DevicePointer(), size, temperature, indices.DevicePointer()));
+    }
+};
+
+struct Sort : Module { // src/Sort.cs
+    using Module::Module;
+    void Forward(DeviceVariable<Half>& logits, DeviceVariable<int>& indices, int size)
+    {
+        Check(llama2_sort(logits.DevicePointer(), indices.DevicePointer(), size));
+    }
+};
+
+struct CumulativeSum : Module { // src/CumulativeSum.cs
+    using Module::Module;
+    void Forward(DeviceVariable<Half>& logits, int size) { Check(llama2_cumulative_sum(logits.DevicePointer(), size)); }
+};
+
+struct SampleTopP : Module { // src/SampleTopP.cs
+    using Module::Module;
+    void Forward(DeviceVariable<Half>& logits, DeviceVariable<int>& indices, int size, float threshold,
+                 DeviceVariable<int>& tokens, int nextPos)
+    {
+        Check(llama2_sample_top_p(logits.DevicePointer(), indices.DevicePointer(), size, threshold, tokens.DevicePointer(),
+                                  nextPos));
+    }
+};
+
+// ---------------------------------------------------------------- src/Sampler.cs
 class Sampler {
   public:
-    Sampler(const Config& config, RunState& runstate) : config_(config), runstate_(runstate), argmax_(&config_) {}
+    Sampler(const Config& config, RunState& runstate, float temperature, float topP, uint64_t seed)
+        : config_(config), runstate_(runstate), temperature_(temperature), topP_(topP), seed_(seed), argmax_(&config_),
+          softmax_(&config_), cumulativeSum_(&config_), sampleTopP_(&config_), sort_(&config_)
+    {
+    }
+    float Temperature() const { return temperature_; }
+    float TopP() const { return topP_; }
+    // The reference draws from an unseeded System.Random (:24, :42); here the coin of a position is the
+    // library's seeded stream, so a run can be reproduced (and matches llama2_decode_run_sampled).
+    float Coin(int nextPosition) const { return llama2_sampler_coin(seed_, nextPosition); }
     int Sample(int nextPosition, bool generateToken)
     {
-        argmax_.Forward(runstate_.logits, config_.vocab_size, runstate_.tokens, nextPosition, generateToken); // :44-47
-        return runstate_.tokens[nextPosition];                                                               // :69
+        const float coin = Coin(nextPosition); // :42
+        RunState& rs = runstate_;
+        const int n = config_.vocab_size;
+        if (temperature_ == 0.0f || !generateToken) {
+            argmax_.Forward(rs.logits, n, rs.tokens, nextPosition, generateToken); // :44-47
+        } else {
+            softmax_.Forward(rs.logits, n, temperature_, rs.indices); // :50
+            float threshold;
+            if (topP_ <= 0 || topP_ >= 1) {
+                threshold = coin; // :53-55
+            } else {
+                sort_.Forward(rs.logits, rs.indices, n); // :59
+                threshold = coin * topP_;                // :61
+            }
+            cumulativeSum_.Forward(rs.logits, n);                                              // :64
+            sampleTopP_.Forward(rs.logits, rs.indices, n, threshold, rs.tokens, nextPosition); // :66
+        }
+        return rs.tokens[nextPosition]; // :69
     }
 
   private:
     Config config_;
     RunState& runstate_;
+    float temperature_, topP_;
+    uint64_t seed_;
     Argmax argmax_;
+    SoftmaxLogits softmax_;
+    CumulativeSum cumulativeSum_;
+    SampleTopP sampleTopP_;
+    Sort sort_;
 };
 
 // ---------------------------------------------------------------- src/ITransformer.cs, src/Transformer.cs
@@ -440,7 +504,9 @@ class Transformer : public ITransformer {
     enum Mode { HostLoop = -1, Modules = LLAMA2_DECODE_MODULES, Fused = LLAMA2_DECODE_FUSED,
                 FusedGraph = LLAMA2_DECODE_FUSED | LLAMA2_DECODE_GRAPH };
 
-    explicit Transformer(const std::string& modelPath, Mode mode = HostLoop, bool stopOnSpecial = true)
+    // temperature 0 is greedy decoding; the reference's defaults are temperature 0.5, topP 0.9 (:42)
+    explicit Transformer(const std::string& modelPath, Mode mode = HostLoop, bool stopOnSpecial = true,
+                         float temperature = 0.0f, float topP = 0.9f, uint64_t seed = 0)
         : stopOnSpecial_(stopOnSpecial)
     {
         Check(llama2_init(0)); // new CudaContext(deviceID), :48-49
@@ -451,7 +517,7 @@ class Transformer : public ITransformer {
             throw NotImplementedException("Differing kvDim dimention not currently supported.");
         weights = std::make_unique<TransformerWeights>(config, file);
         runstate = std::make_unique<RunState>(config, kvDim);
-        sampler = std::make_unique<Sampler>(config, *runstate);
+        sampler = std::make_unique<Sampler>(config, *runstate, temperature, topP, seed);
         embedding = Embedding(&config);
         rmsNorm = RMSNorm(&config);
         qkvMatVec = QKVMatVec(&config);
@@ -532,7 +598,8 @@ class Transformer : public ITransformer {
     {
         if (decoder_) {
             int token = 0;
-            Check(llama2_decode_sample(decoder_, nextPos, generateToken ? 1 : 0, &token));
+            Check(llama2_decode_sample_top_p(decoder_, nextPos, generateToken ? 1 : 0, sampler->Temperature(),
+                                             sampler->TopP(), sampler->Coin(nextPos), &token));
             return token;
         }
         return sampler->Sample(nextPos, generateToken);

@@ -59,6 +59,16 @@ __attribute__((visibility("default"))) int l2h_transformer_open(const char* path
     return guarded([&] { *handle = new Transformer(path, static_cast<Transformer::Mode>(mode), stop_on_special != 0); });
 }
 
+__attribute__((visibility("default"))) int l2h_transformer_open_sampled(const char* path, int mode, int stop_on_special,
+                                                                        float temperature, float top_p,
+                                                                        unsigned long long seed, void** handle)
+{
+    *handle = nullptr;
+    return guarded([&] {
+        *handle = new Transformer(path, static_cast<Transformer::Mode>(mode), stop_on_special != 0, temperature, top_p, seed);
+    });
+}
+
 __attribute__((visibility("default"))) int l2h_transformer_generate(void* handle, const int* prompt, int n_prompt, int steps,
                                                                     int* out, int* n_out)
 {

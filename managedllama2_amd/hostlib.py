@@ -27,6 +27,8 @@ def load():
         lib.l2h_last_error.restype = C.c_char_p
         lib.l2h_check_model_file.argtypes = [C.c_char_p]
         lib.l2h_transformer_open.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
+        lib.l2h_transformer_open_sampled.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_float, C.c_float,
+                                                     C.c_ulonglong, C.POINTER(C.c_void_p)]
         lib.l2h_transformer_generate.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_int, C.POINTER(C.c_int),
                                                  C.POINTER(C.c_int)]
         lib.l2h_transformer_logits.argtypes = [C.c_void_p, C.POINTER(C.c_uint16), C.c_int]
@@ -48,9 +50,14 @@ def check_model_file(path):
 class Transformer:
     """libLlama2::Transformer (ITransformer on token ids)."""
 
-    def __init__(self, model_path, mode=HOST_LOOP, stop_on_special=True):
+    def __init__(self, model_path, mode=HOST_LOOP, stop_on_special=True, temperature=0.0, top_p=0.9, seed=0):
         self._h = C.c_void_p()
-        _check(load().l2h_transformer_open(model_path.encode(), mode, 1 if stop_on_special else 0, C.byref(self._h)))
+        if temperature == 0.0:
+            _check(load().l2h_transformer_open(model_path.encode(), mode, 1 if stop_on_special else 0,
+                                               C.byref(self._h)))
+        else:
+            _check(load().l2h_transformer_open_sampled(model_path.encode(), mode, 1 if stop_on_special else 0,
+                                                       temperature, top_p, seed, C.byref(self._h)))
 
     def Generate(self, prompt_tokens, steps):
         prompt = (C.c_int * len(prompt_tokens))(*[int(t) for t in prompt_tokens])

@@ -132,3 +132,31 @@ class Embedding(Module):
 
     def Forward(self, output, table, size, tokens, pos):
         capi.call("llama2_embedding", output.ptr, table.ptr, size, tokens.ptr, pos)
+
+
+class SoftmaxLogits(Module):
+    """src/SoftmaxLogits.cs:5-16"""
+
+    def Forward(self, logits, size, temperature, indices):
+        capi.call("llama2_softmax_logits", logits.ptr, size, temperature, indices.ptr)
+
+
+class Sort(Module):
+    """src/Sort.cs:5-16"""
+
+    def Forward(self, logits, indices, size):
+        capi.call("llama2_sort", logits.ptr, indices.ptr, size)
+
+
+class CumulativeSum(Module):
+    """src/CumulativeSum.cs:5-16"""
+
+    def Forward(self, logits, size):
+        capi.call("llama2_cumulative_sum", logits.ptr, size)
+
+
+class SampleTopP(Module):
+    """src/SampleTopP.cs:5-16"""
+
+    def Forward(self, logits, indices, size, threshold, tokens, nextPos):
+        capi.call("llama2_sample_top_p", logits.ptr, indices.ptr, size, threshold, tokens.ptr, nextPos)

@@ -1,6 +1,5 @@
 """Host-side orchestration of the decode path, mirroring src/Transformer.cs,
-src/TransformerWeights.cs, src/RunState.cs and the greedy branch of
-src/Sampler.cs over the C ABI.  Text (tokenizer, chat templating) is outside
+src/TransformerWeights.cs, src/RunState.cs and src/Sampler.cs over the C ABI.  Text (tokenizer, chat templating) is outside
 this path: Generate takes and yields token ids.
 """
 import ctypes as C
@@ -10,8 +9,8 @@ import numpy as np
 
 from . import capi
 from .device import DeviceVariable, QWeight, init
-from .modules import (Argmax, Embedding, MatVec, MatVecResidual, MatVecStrided, MatVecSwiGLU, QKVMatVec,
-                      RMSNorm, RoPERotation, Softmax, VecMat)
+from .modules import (Argmax, CumulativeSum, Embedding, MatVec, MatVecResidual, MatVecStrided, MatVecSwiGLU,
+                      QKVMatVec, RMSNorm, RoPERotation, SampleTopP, Softmax, SoftmaxLogits, Sort, VecMat)
 
 
 def make_config(d):
@@ -84,23 +83,43 @@ class RunState:
         self.keyCache = DeviceVariable.zeros(half, config.n_layers * config.seq_len * kvDim)
         self.valueCache = DeviceVariable.zeros(half, config.n_layers * config.seq_len * kvDim)
         self.tokens = DeviceVariable.zeros(np.int32, config.seq_len + 1)
+        self.indices = DeviceVariable(np.int32, config.vocab_size)
 
     def struct(self):
         return capi.RunState(self.x.ptr, self.xb.ptr, self.h.ptr, self.q.ptr, self.attention.ptr,
-                             self.logits.ptr, self.keyCache.ptr, self.valueCache.ptr, self.tokens.ptr)
+                             self.logits.ptr, self.keyCache.ptr, self.valueCache.ptr, self.tokens.ptr,
+                             self.indices.ptr)
 
 
 class Sampler:
-    """Greedy branch of src/Sampler.cs:40-47,69 (temperature == 0)."""
+    """src/Sampler.cs:5-72.  `random` supplies the coin (a callable returning a
+    float in [0, 1)); the reference draws it from an unseeded System.Random."""
 
-    def __init__(self, config, runstate):
+    def __init__(self, config, runstate, temperature=0.0, topP=0.9, random=None):
         self.config, self.runstate = config, runstate
+        self.temperature, self.topP = float(temperature), float(topP)
+        self.random = random if random is not None else np.random.default_rng().random
         self.argmax = Argmax(config)
+        self.softmax = SoftmaxLogits(config)
+        self.cumulativeSum = CumulativeSum(config)
+        self.sampleTopP = SampleTopP(config)
+        self.sort = Sort(config)
 
     def Sample(self, nextPosition, generateToken):
-        self.argmax.Forward(self.runstate.logits, self.config.vocab_size, self.runstate.tokens, nextPosition,
-                            generateToken)
-        return int(self.runstate.tokens[nextPosition])
+        coin = float(np.float32(self.random()))
+        rs, n = self.runstate, self.config.vocab_size
+        if self.temperature == 0.0 or not generateToken:
+            self.argmax.Forward(rs.logits, n, rs.tokens, nextPosition, generateToken)
+        else:
+            self.softmax.Forward(rs.logits, n, self.temperature, rs.indices)
+            if self.topP <= 0 or self.topP >= 1:
+                threshold = coin
+            else:
+                self.sort.Forward(rs.logits, rs.indices, n)
+                threshold = float(np.float32(coin) * np.float32(self.topP))
+            self.cumulativeSum.Forward(rs.logits, n)
+            self.sampleTopP.Forward(rs.logits, rs.indices, n, threshold, rs.tokens, nextPosition)
+        return int(rs.tokens[nextPosition])
 
 
 class Transformer:
@@ -108,7 +127,7 @@ class Transformer:
     from the host exactly like the C# Forward; a capi.DECODE_* value hands the
     step to llama2_decode_forward."""
 
-    def __init__(self, config_dict, host_weights, mode=None, device=0):
+    def __init__(self, config_dict, host_weights, mode=None, device=0, temperature=0.0, topP=0.9, random=None):
         init(device)
         self.config = make_config(config_dict)
         c = self.config
@@ -119,7 +138,7 @@ class Transformer:
             raise NotImplementedError("Differing kvDim dimention not currently supported.")  # Transformer.cs:55-56
         self.weights = TransformerWeights(c, host_weights)
         self.runstate = RunState(c, self.kvDim)
-        self.sampler = Sampler(c, self.runstate)
+        self.sampler = Sampler(c, self.runstate, temperature, topP, random)
         self.embedding = Embedding(c)
         self.rmsNorm = RMSNorm(c)
         self.qkvMatVec = QKVMatVec(c)
@@ -161,7 +180,9 @@ class Transformer:
     def Sample(self, nextPos, generateToken):
         if self._decoder is not None:
             tok = C.c_int()
-            capi.call("llama2_decode_sample", self._decoder, nextPos, 1 if generateToken else 0, C.byref(tok))
+            sp = self.sampler
+            capi.call("llama2_decode_sample_top_p", self._decoder, nextPos, 1 if generateToken else 0,
+                      sp.temperature, sp.topP, float(np.float32(sp.random())), C.byref(tok))
             return tok.value
         return self.sampler.Sample(nextPos, generateToken)
 

@@ -1,0 +1,174 @@
+"""Sampler.Sample with temperature and top-p (src/Sampler.cs:40-70) inside the
+decode loop: the host loop over the four sampler modules, the decoder's
+one-launch sampler, the device-resident sampling loop (eager and hipGraph) and
+the C++ host must all pick the same tokens from the same coins, and agree with
+the CPU oracle teacher-forced on the GPU's history."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from managedllama2_amd import capi, hostlib, modelfile, synth
+from managedllama2_amd.transformer import Transformer
+
+pytestmark = pytest.mark.gpu
+
+CFG = dict(dim=512, hidden_dim=1408, n_layers=3, n_heads=4, n_kv_heads=4, vocab_size=1000, seq_len=64, rope_theta=10000.0)
+FUSED = capi.DECODE_FUSED
+FUSED_GRAPH = capi.DECODE_FUSED | capi.DECODE_GRAPH
+T, TOP_P, SEED = 0.7, 0.9, 20240607
+
+
+def lib_coin(seed, pos):
+    return float(capi.load().llama2_sampler_coin(seed, pos))
+
+
+class CoinStream:
+    """The seeded coin of a position, handed to the host Sampler one call at a time."""
+
+    def __init__(self, seed):
+        self.seed, self.pos = seed, 0
+
+    def __call__(self):
+        return lib_coin(self.seed, self.pos)
+
+
+def stepwise(model, mode, prompt, steps, temperature=T, top_p=TOP_P, seed=SEED):
+    coins = CoinStream(seed)
+    t = Transformer(dict(CFG), model, mode=mode, temperature=temperature, topP=top_p, random=coins)
+    t.runstate.tokens.copy_to_device(np.array(prompt, np.int32))
+    out = []
+    for pos in range(steps):
+        t.Forward(pos, pos + 1)
+        coins.pos = pos + 1
+        gen = pos + 1 >= len(prompt)
+        tok = t.Sample(pos + 1, gen)
+        out.append(tok)
+    t.close()
+    return out
+
+
+def test_coin_is_the_oracles(oracle):
+    for seed in (0, 1, SEED, 2 ** 63 + 12345):
+        for pos in (0, 1, 2, 100, 4095):
+            assert lib_coin(seed, pos) == oracle.coin(seed, pos)
+    c = np.array([lib_coin(SEED, p) for p in range(2000)])
+    assert c.min() >= 0 and c.max() < 1 and abs(c.mean() - 0.5) < 0.03
+
+
+def test_decoder_sampler_equals_module_sampler():
+    """Host loop over the four sampler modules == decoder's one-launch sampler (the module-by-module
+    forward gives bit-identical logits in both, so every token must agree)."""
+    model = synth.random_model(CFG, seed=33, rms_random=True)
+    prompt = [int(t) for t in synth.rng_for(601).integers(3, CFG["vocab_size"], 4)]
+    a = stepwise(model, None, prompt, 40)
+    b = stepwise(model, capi.DECODE_MODULES, prompt, 40)
+    assert a == b
+    assert a[:3] == prompt[1:]
+    assert len(set(a[3:])) > 10  # it samples, it is not stuck
+    greedy = stepwise(model, None, prompt, 40, temperature=0.0)
+    assert greedy != a
+
+
+@pytest.mark.parametrize("mode", [capi.DECODE_MODULES, FUSED, FUSED_GRAPH])
+def test_device_resident_sampling_loop(mode):
+    model = synth.random_model(CFG, seed=34, rms_random=True)
+    prompt = [int(t) for t in synth.rng_for(602).integers(3, CFG["vocab_size"], 5)]
+    want = stepwise(model, mode, prompt, 45)
+    t = Transformer(dict(CFG), model, mode=mode)
+    t.runstate.tokens.copy_to_device(np.array(prompt, np.int32))
+    capi.call("llama2_decode_run_sampled", t._decoder, 0, 30, len(prompt), T, TOP_P, SEED)
+    capi.call("llama2_decode_run_sampled", t._decoder, 30, 15, len(prompt), T, TOP_P, SEED)  # continue
+    got = list(t.runstate.tokens.to_host(46)[1:])
+    assert got == want
+    # other parameters: the captured step is rebuilt; plain inverse-CDF sampling (top_p = 1); another seed
+    want2 = stepwise(model, mode, prompt, 20, temperature=1.3, top_p=1.0, seed=7)
+    t.runstate.tokens.copy_to_device(np.array(prompt + [0] * 40, np.int32))
+    capi.call("llama2_decode_run_sampled", t._decoder, 0, 20, len(prompt), 1.3, 1.0, 7)
+    assert list(t.runstate.tokens.to_host(21)[1:]) == want2 and want2 != want[:20]
+    # temperature 0 is the greedy loop
+    t.runstate.tokens.copy_to_device(np.array(prompt + [0] * 40, np.int32))
+    capi.call("llama2_decode_run_sampled", t._decoder, 0, 20, len(prompt), 0.0, TOP_P, SEED)
+    g1 = list(t.runstate.tokens.to_host(21)[1:])
+    t.runstate.tokens.copy_to_device(np.array(prompt + [0] * 40, np.int32))
+    capi.call("llama2_decode_run", t._decoder, 0, 20, len(prompt))
+    assert g1 == list(t.runstate.tokens.to_host(21)[1:])
+    t.close()
+
+
+def test_graph_replays_of_the_sampling_step_are_stable():
+    """The same run twice, with eager work and synchronisation in between."""
+    model = synth.random_model(CFG, seed=35)
+    prompt = [5, 6, 7]
+    t = Transformer(dict(CFG), model, mode=FUSED_GRAPH)
+    runs = []
+    for rep in range(3):
+        t.runstate.tokens.copy_to_device(np.array(prompt + [0] * 40, np.int32))
+        capi.call("llama2_decode_run_sampled", t._decoder, 0, 25, len(prompt), T, TOP_P, SEED)
+        runs.append(list(t.runstate.tokens.to_host(26)))
+        capi.call("llama2_memset", t.runstate.logits.ptr, 0, 16)
+    assert runs[0] == runs[1] == runs[2]
+    t.close()
+
+
+def test_sampled_tokens_against_the_oracle(oracle):
+    """Teacher-forced: the oracle replays each step on the GPU's token history and samples with the same
+    coin.  The logits of the two sides differ by fp16 rounding flips (see test_gpu_transformer.py); with a
+    vocabulary of 1000 near-equal probabilities that is enough to swap neighbours in the sorted order, so
+    the token at the sampled RANK may differ while the rank itself does not.  Hence two checks: the GPU's
+    token must occupy, in the oracle's sorted distribution, a slice of cumulative probability that
+    contains the threshold coin * top_p up to 0.02; and a fair share of the tokens agree exactly."""
+    model = synth.random_model(CFG, seed=36, rms_random=True)
+    prompt = [int(t) for t in synth.rng_for(603).integers(3, CFG["vocab_size"], 4)]
+    steps = 40
+    got = stepwise(model, FUSED_GRAPH, prompt, steps)
+    hm = oracle.HostModel(CFG, model)
+    hm.tokens[:len(prompt)] = prompt
+    agree = generated = 0
+    for pos in range(steps):
+        logits = hm.forward(pos, pos + 1)
+        if pos + 1 >= len(prompt):
+            coin = oracle.coin(SEED, pos + 1)
+            want = oracle.ref_sample(logits, T, TOP_P, coin)
+            generated += 1
+            agree += want == got[pos]
+            p, idx = oracle.ref_sort(*oracle.ref_softmax_logits(logits, T))
+            cdf = np.cumsum(p.astype(np.float64))
+            j = int(np.nonzero(idx == got[pos])[0][0])
+            thr = coin * TOP_P
+            assert cdf[j] - float(p[j]) - 0.02 <= thr <= cdf[j] + 0.02, (pos, got[pos], want, thr, cdf[j])
+            hm.tokens[pos + 1] = got[pos]
+    assert agree >= generated // 3, (agree, generated)
+
+
+def test_rejects_missing_indices_and_bad_temperature():
+    model = synth.random_model(CFG, seed=35)
+    t = Transformer(dict(CFG), model, mode=None)
+    w, s = t.weights.struct(), t.runstate.struct()
+    s.indices = None
+    cfg = capi.Config(*[CFG[k] for k in ("dim", "hidden_dim", "n_layers", "n_heads", "n_kv_heads", "vocab_size", "seq_len")],
+                      CFG["rope_theta"])
+    h = C.c_void_p()
+    capi.call("llama2_decode_create", C.byref(h), C.byref(cfg), C.byref(w), C.byref(s), capi.DECODE_MODULES)
+    tok = C.c_int()
+    assert capi.raw("llama2_decode_sample_top_p", h, 1, 1, 0.7, 0.9, 0.5, C.byref(tok)) == capi.ERR_INVALID_ARGUMENT
+    assert "indices" in capi.last_error()
+    assert capi.raw("llama2_decode_run_sampled", h, 0, 2, 1, -1.0, 0.9, 1) == capi.ERR_INVALID_ARGUMENT
+    # greedy sampling needs no indices buffer
+    t.runstate.tokens.copy_to_device(np.array([5], np.int32))
+    capi.call("llama2_decode_forward", h, 0, 1)
+    capi.call("llama2_decode_sample_top_p", h, 1, 1, 0.0, 0.9, 0.5, C.byref(tok))
+    assert 0 <= tok.value < CFG["vocab_size"]
+    capi.call("llama2_decode_destroy", h)
+
+
+@pytest.mark.parametrize("host_mode,py_mode", [(hostlib.HOST_LOOP, None), (hostlib.FUSED_GRAPH, FUSED_GRAPH)])
+def test_cpp_host_samples_the_same_tokens(tmp_path, host_mode, py_mode):
+    path = str(tmp_path / "model.bin")
+    model = synth.random_model(CFG, seed=37, rms_random=True)
+    modelfile.write_model(path, CFG, model)
+    prompt = [int(t) for t in synth.rng_for(604).integers(3, CFG["vocab_size"], 5)]
+    t = hostlib.Transformer(path, host_mode, stop_on_special=False, temperature=T, top_p=TOP_P, seed=SEED)
+    got = t.Generate(prompt, 30)
+    t.close()
+    assert got == stepwise(model, py_mode, prompt, 30)
