@@ -58,14 +58,14 @@ def main():
     ap.add_argument("--steps", type=int, default=3200)
     ap.add_argument("--warmup", type=int, default=320)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
-    ap.add_argument("--only", default="", help="comma list of legs: set,kernel,attn,decode,cpu (default all)")
+    ap.add_argument("--only", default="", help="comma list of legs: set,kernel,calib,attn,decode,sampler,cpu (default: all but calib)")
     ap.add_argument("--decode-mode", default="fused_graph", choices=["modules", "fused", "fused_graph"])
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (batch-1 decode has no cross-GPU exchange to measure); "
             "--gpus %d is not supported" % args.gpus)
         sys.exit(2)
-    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "attn", "decode", "cpu"}
+    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "attn", "decode", "sampler", "cpu"}
 
     from managedllama2_amd import capi, synth
     from managedllama2_amd.device import DeviceVariable, init
@@ -298,6 +298,55 @@ def main():
         log("decode: %.1f tok/s (%.3f ms/token, %.0f GB/s = %.1f%% of peak; ceiling %.0f tok/s)" %
             (tok_s, ms / steps, bytes_tok * tok_s / 1e9, 100 * bytes_tok * tok_s / 1e9 / HBM_PEAK_GBPS,
              HBM_PEAK_GBPS * 1e9 / bytes_tok))
+
+    if "sampler" in legs:
+        # Sampler.Sample with the reference's defaults (temperature 0.5, top-p 0.9) on 32000 logits:
+        # the four module launches, the one-launch sampler, and the device-resident decode loop with it
+        vocab = cfg["vocab_size"]
+        logits_host = synth.normal_f16(synth.rng_for(6), vocab, 2.0)
+        lg, idx = DeviceVariable.from_host(logits_host), DeviceVariable.zeros(np.int32, vocab)
+        src = DeviceVariable.from_host(logits_host)
+        tok = DeviceVariable.zeros(np.int32, 2)
+        temp, top_p = 0.5, 0.9
+        sampler = {}
+
+        def timed(name, fn):
+            graph = capture(lambda i: (capi.call("llama2_memcpy_d2d", lg.ptr, src.ptr, vocab * 2), fn()), 16)
+            base = capture(lambda i: capi.call("llama2_memcpy_d2d", lg.ptr, src.ptr, vocab * 2), 16)
+            for g in (graph, base):
+                capi.call("llama2_graph_launch", g)
+            us = 1e3 * (timed_replays(graph, 20) - timed_replays(base, 20)) / (20 * 16)
+            capi.call("llama2_graph_destroy", graph)
+            capi.call("llama2_graph_destroy", base)
+            sampler[name] = round(us, 2)
+
+        timed("softmax_logits_us", lambda: capi.call("llama2_softmax_logits", lg.ptr, vocab, temp, idx.ptr))
+        timed("sort_us", lambda: capi.call("llama2_sort", lg.ptr, idx.ptr, vocab))
+        timed("cumulative_sum_us", lambda: capi.call("llama2_cumulative_sum", lg.ptr, vocab))
+        timed("sample_top_p_us", lambda: capi.call("llama2_sample_top_p", lg.ptr, idx.ptr, vocab, 0.45, tok.ptr, 1))
+        timed("four_modules_us", lambda: (capi.call("llama2_softmax_logits", lg.ptr, vocab, temp, idx.ptr),
+                                          capi.call("llama2_sort", lg.ptr, idx.ptr, vocab),
+                                          capi.call("llama2_cumulative_sum", lg.ptr, vocab),
+                                          capi.call("llama2_sample_top_p", lg.ptr, idx.ptr, vocab, 0.45, tok.ptr, 1)))
+        timed("one_launch_us", lambda: capi.call("llama2_sample", lg.ptr, idx.ptr, vocab, temp, top_p, 0.5, tok.ptr, 1))
+        n_prompt, n_gen = 128, 256
+        steps = n_prompt + n_gen - 1
+        prompt = synth.rng_for(5).integers(3, vocab, n_prompt).astype(np.int32)
+        model.runstate.tokens.copy_to_device(prompt)
+        capi.call("llama2_decode_run_sampled", model._decoder, 0, 16, n_prompt, temp, top_p, 1)  # warm-up
+        capi.call("llama2_sync")
+        ev.start()
+        capi.call("llama2_decode_run_sampled", model._decoder, 0, steps, n_prompt, temp, top_p, 1)
+        ms = ev.stop_ms()
+        sampler["decode_tokens_per_s"] = round(steps / (ms * 1e-3), 1)
+        sampler["decode_ms_per_token"] = round(ms / steps, 4)
+        sampler["temperature"], sampler["top_p"] = temp, top_p
+        result["sampler"] = sampler
+        log("sampler (32000 logits, T=0.5, top-p 0.9): softmax %.1f + sort %.1f + cumsum %.1f + pick %.1f us; "
+            "4 launches %.1f us, one launch %.1f us; sampled decode %.1f tok/s" %
+            (sampler["softmax_logits_us"], sampler["sort_us"], sampler["cumulative_sum_us"],
+             sampler["sample_top_p_us"], sampler["four_modules_us"], sampler["one_launch_us"],
+             sampler["decode_tokens_per_s"]))
 
     if "cpu" in legs and args.cpu_seconds > 0:
         from oracle import oracle

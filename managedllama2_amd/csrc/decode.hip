@@ -316,25 +316,48 @@ __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, in
 // Sampler.Sample's stochastic branch (src/Sampler.cs:48-67) against the device
 // state: the token at pos+1 is drawn with the coin of (seed, pos+1) iff
 // pos+1 >= n_prompt; then the position advances like in argmax_step_kernel.
-template <int CH>
-__global__ __launch_bounds__(kSampBlock) void sample_step_kernel(uint16_t* logits, int* indices, int size, int* tokens,
-                                                                 int* state, uint16_t* keys2, int* values2,
-                                                                 float temperature, float top_p,
-                                                                 unsigned long long seed, float theta)
+struct SampleStepArgs {
+    uint16_t* logits;
+    int* indices;
+    int size;
+    int* tokens;
+    int* state;
+    uint16_t* keys2; // second buffer of the global-memory sort (vocabularies beyond kSortLdsItems)
+    int* values2;
+    float temperature, top_p;
+    unsigned long long seed;
+    float theta;
+};
+
+template <bool LDS_SORT>
+__device__ __forceinline__ void sample_step(const SampleStepArgs& a, SamplerLds& lds, SortLds* buf)
 {
-    __shared__ SamplerLds lds;
-    const int pos0 = state[0], n_prompt = state[1], advance0 = state[2];
+    const int pos0 = a.state[0], n_prompt = a.state[1], advance0 = a.state[2];
     if (advance0 && threadIdx.x >= 64 && threadIdx.x < 64 + kRopeHeadSize / 2)
-        write_rope_table(state, threadIdx.x - 64, pos0 + 1, theta); // for the next step
+        write_rope_table(a.state, threadIdx.x - 64, pos0 + 1, a.theta); // for the next step
     if (pos0 + 1 >= n_prompt) { // uniform over the workgroup
-        const int token = sample_dev<CH>(logits, indices, size, temperature, top_p, sampler_coin(seed, pos0 + 1),
-                                         keys2, values2, lds);
+        const float coin = sampler_coin(a.seed, pos0 + 1);
+        const int token = sample_dev<LDS_SORT ? 4 : 8, LDS_SORT>(a.logits, a.indices, a.size, a.temperature, a.top_p,
+                                                                 coin, a.keys2, a.values2, lds, buf);
         if (threadIdx.x == 0)
-            tokens[pos0 + 1] = token;
+            a.tokens[pos0 + 1] = token;
     }
     __syncthreads(); // every thread has read the state
     if (threadIdx.x == 0 && advance0)
-        state[0] = pos0 + 1;
+        a.state[0] = pos0 + 1;
+}
+
+__global__ __launch_bounds__(kSampBlock) void sample_step_kernel(SampleStepArgs a)
+{
+    __shared__ SamplerLds lds;
+    __shared__ SortLds buf;
+    sample_step<true>(a, lds, &buf);
+}
+
+__global__ __launch_bounds__(kSampBlock) void sample_step_big_kernel(SampleStepArgs a)
+{
+    __shared__ SamplerLds lds;
+    sample_step<false>(a, lds, nullptr);
 }
 
 } // namespace l2
@@ -491,15 +514,12 @@ int launch_argmax_step(llama2_decoder* d)
 
 int launch_sample_step(llama2_decoder* d, float temperature, float top_p, unsigned long long seed)
 {
-    const int size = d->cfg.vocab_size;
-    if (size <= 4 * 8 * kSampBlock)
-        hipLaunchKernelGGL(sample_step_kernel<4>, dim3(1), dim3(kSampBlock), 0, ctx().stream, d->s.logits, d->s.indices,
-                           size, d->s.tokens, d->state, ctx().sort_keys, ctx().sort_values, temperature, top_p, seed,
-                           d->cfg.rope_theta);
+    SampleStepArgs a{d->s.logits, d->s.indices, d->cfg.vocab_size, d->s.tokens, d->state, ctx().sort_keys,
+                     ctx().sort_values, temperature, top_p, seed, d->cfg.rope_theta};
+    if (a.size <= kSortLdsItems)
+        hipLaunchKernelGGL(sample_step_kernel, dim3(1), dim3(kSampBlock), 0, ctx().stream, a);
     else
-        hipLaunchKernelGGL(sample_step_kernel<8>, dim3(1), dim3(kSampBlock), 0, ctx().stream, d->s.logits, d->s.indices,
-                           size, d->s.tokens, d->state, ctx().sort_keys, ctx().sort_values, temperature, top_p, seed,
-                           d->cfg.rope_theta);
+        hipLaunchKernelGGL(sample_step_big_kernel, dim3(1), dim3(kSampBlock), 0, ctx().stream, a);
     L2_LAUNCH_CHECK("sample_step_kernel");
     return LLAMA2_OK;
 }

@@ -23,6 +23,13 @@ __global__ __launch_bounds__(kSampBlock) void sort_kernel(uint16_t* keys, int* v
     sort_dev<CH>(keys, values, size, keys2, values2, lds);
 }
 
+__global__ __launch_bounds__(kSampBlock) void sort_lds_kernel(uint16_t* keys, int* values, int size)
+{
+    __shared__ SamplerLds lds;
+    __shared__ SortLds buf;
+    sort_lds_dev<false>(keys, values, size, lds, buf);
+}
+
 template <int CH>
 __global__ __launch_bounds__(kSampBlock) void cumulative_sum_kernel(uint16_t* values, int size)
 {
@@ -40,13 +47,22 @@ __global__ __launch_bounds__(kSampBlock) void sample_top_p_kernel(const uint16_t
         result[pos] = token;
 }
 
-template <int CH>
 __global__ __launch_bounds__(kSampBlock) void sample_kernel(uint16_t* logits, int* indices, int size, float temperature,
-                                                            float top_p, float coin, int* result, int pos,
-                                                            uint16_t* keys2, int* values2)
+                                                            float top_p, float coin, int* result, int pos)
 {
     __shared__ SamplerLds lds;
-    const int token = sample_dev<CH>(logits, indices, size, temperature, top_p, coin, keys2, values2, lds);
+    __shared__ SortLds buf;
+    const int token = sample_dev<4, true>(logits, indices, size, temperature, top_p, coin, nullptr, nullptr, lds, &buf);
+    if (threadIdx.x == 0)
+        result[pos] = token;
+}
+
+__global__ __launch_bounds__(kSampBlock) void sample_big_kernel(uint16_t* logits, int* indices, int size,
+                                                                float temperature, float top_p, float coin, int* result,
+                                                                int pos, uint16_t* keys2, int* values2)
+{
+    __shared__ SamplerLds lds;
+    const int token = sample_dev<8, false>(logits, indices, size, temperature, top_p, coin, keys2, values2, lds, nullptr);
     if (threadIdx.x == 0)
         result[pos] = token;
 }
@@ -102,7 +118,10 @@ int llama2_sort(llama2_half* keys, int* values, int size)
     L2_CHECK(keys && values, "%s: null pointer", fn);
     L2_TRY(check_sampler_size(fn, size));
     L2_CHECK(aligned(keys, 16) && aligned(values, 16), "%s: keys and values must be 16-byte aligned", fn);
-    L2_SAMPLER_LAUNCH(sort_kernel, size, keys, values, size, ctx().sort_keys, ctx().sort_values);
+    if (size <= kSortLdsItems)
+        hipLaunchKernelGGL(sort_lds_kernel, dim3(1), dim3(kSampBlock), 0, ctx().stream, keys, values, size);
+    else
+        L2_SAMPLER_LAUNCH(sort_kernel, size, keys, values, size, ctx().sort_keys, ctx().sort_values);
     L2_LAUNCH_CHECK(fn);
     return LLAMA2_OK;
 }
@@ -143,8 +162,12 @@ int llama2_sample(llama2_half* logits, int* indices, int size, float temperature
              static_cast<double>(temperature));
     L2_CHECK(pos >= 0, "%s: pos=%d is negative", fn, pos);
     L2_CHECK(aligned(logits, 16) && aligned(indices, 16), "%s: logits and indices must be 16-byte aligned", fn);
-    L2_SAMPLER_LAUNCH(sample_kernel, size, logits, indices, size, temperature, top_p, coin, result, pos,
-                      ctx().sort_keys, ctx().sort_values);
+    if (size <= kSortLdsItems)
+        hipLaunchKernelGGL(sample_kernel, dim3(1), dim3(kSampBlock), 0, ctx().stream, logits, indices, size, temperature,
+                           top_p, coin, result, pos);
+    else
+        hipLaunchKernelGGL(sample_big_kernel, dim3(1), dim3(kSampBlock), 0, ctx().stream, logits, indices, size,
+                           temperature, top_p, coin, result, pos, ctx().sort_keys, ctx().sort_values);
     L2_LAUNCH_CHECK(fn);
     return LLAMA2_OK;
 }

@@ -317,6 +317,169 @@ __device__ __forceinline__ void sort_dev(uint16_t* keys, int* values, int size, 
     }
 }
 
+// The same sort with every pass inside LDS, for up to kSortLdsItems items (a
+// 32000-entry vocabulary fits).  Scattering 2- and 4-byte items to global memory
+// from one compute unit costs one cache-line transaction per lane and made the
+// sort above take 140 us for 32000 items; in LDS a scatter is a bank access.
+// An item is (rank << 16) | original position; a thread owns 32 consecutive
+// positions, kept in registers between passes.  Slot p lives at word
+// p ^ ((p >> 5) & 31), so a thread reading its 32 consecutive slots and the 64
+// lanes of a wavefront reading slot k of 64 threads both spread over all banks.
+constexpr int kSortLdsThreads = 1008;
+constexpr int kSortLdsItems = kSortLdsThreads * 32; // 32256: data + counters fill the 160 KB of LDS
+
+struct SortLds {
+    uint32_t item[kSortLdsItems];
+};
+
+__device__ __forceinline__ int sort_slot(int p) { return p ^ ((p >> 5) & 31); }
+__device__ __forceinline__ uint16_t sort_key_of_rank(uint32_t rank)
+{
+    return static_cast<uint16_t>((rank & 0x8000u) ? rank ^ 0x8000u : ~rank);
+}
+
+// IDENTITY: values[i] == i on entry (as softmax_logits leaves them), so the
+// sorted payload is the original position itself and no gather is needed.
+template <bool IDENTITY>
+__device__ __forceinline__ void sort_lds_dev(uint16_t* keys, int* values, int size, SamplerLds& lds, SortLds& buf)
+{
+    const int first = threadIdx.x * 32;
+    const bool active = first < size; // threads beyond the (padded) input own nothing
+    uint32_t it[32];
+    if (active) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint16_t kb[8];
+            load_bits8(kb, keys, first + c * 8, size);
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const int idx = first + c * 8 + k;
+                // padding up to the thread's 32 items: smallest rank, behind every real item (stable)
+                it[c * 8 + k] = (idx < size ? sort_rank(kb[k]) << 16 : 0u) | static_cast<uint32_t>(idx);
+            }
+        }
+    }
+    // Between the read-back of one pass and the scatter of the next the item
+    // buffer is idle: its first 16 x 1024 words serve as 32-bit (bucket, thread)
+    // counters, filled with fire-and-forget LDS adds.
+    static_assert(kSortLdsItems >= 16 * kSampBlock, "the counters borrow the item buffer");
+    uint32_t* cnt32 = buf.item;
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 16 + 4 * pass;
+#pragma unroll
+        for (int d = 0; d < 16; ++d)
+            cnt32[d * kSampBlock + threadIdx.x] = 0u;
+        // own words only: no barrier needed before the adds below
+        if (active) {
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                const uint32_t d = 15u - ((it[k] >> shift) & 15u); // bucket 0 = largest digit
+                __hip_atomic_fetch_add(&cnt32[d * kSampBlock + threadIdx.x], 1u, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_WORKGROUP);
+            }
+        }
+        __syncthreads();
+        {
+            // exclusive scan in (bucket, thread) order: 16 consecutive counters per thread
+            const u32x4* mine = reinterpret_cast<const u32x4*>(cnt32 + threadIdx.x * 16);
+            int local[16], total = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const u32x4 c4 = mine[q];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    local[q * 4 + i] = total;
+                    total += static_cast<int>(c4[i]);
+                }
+            }
+            const int before = samp_block_exclusive_scan<int>(total, lds.redi);
+            u32x4* out = reinterpret_cast<u32x4*>(lds.counts + threadIdx.x * 16);
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                u32x4 w;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    w[i] = static_cast<uint32_t>(before + local[q * 8 + 2 * i]) |
+                           (static_cast<uint32_t>(before + local[q * 8 + 2 * i + 1]) << 16);
+                out[q] = w; // 16-bit cursors: positions stay below 32256
+            }
+        }
+        __syncthreads();
+        if (active) {
+            // the cursor of (bucket, thread) is one half of a 32-bit word shared with the neighbouring
+            // thread: an LDS add on the word returns the old cursor and advances it in one operation
+            uint32_t* words = reinterpret_cast<uint32_t*>(lds.counts);
+            const uint32_t one = (threadIdx.x & 1) ? 0x10000u : 1u;
+            const int hshift = (threadIdx.x & 1) * 16;
+#pragma unroll
+            for (int k = 0; k < 32; ++k) {
+                const uint32_t d = 15u - ((it[k] >> shift) & 15u);
+                const uint32_t old = __hip_atomic_fetch_add(&words[(d * kSampBlock + threadIdx.x) >> 1], one,
+                                                            __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                const int at = static_cast<int>((old >> hshift) & 0xFFFFu);
+                buf.item[sort_slot(at)] = it[k];
+                if ((k & 7) == 7)
+                    asm volatile("" ::: "memory"); // at most 8 cursors in flight: keeps the items in registers
+            }
+        }
+        __syncthreads();
+        if (active) {
+#pragma unroll
+            for (int k = 0; k < 32; ++k)
+                it[k] = buf.item[sort_slot(first + k)];
+        }
+        __syncthreads(); // everyone has its items back before the buffer turns into counters again
+    }
+    if (active) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint16_t kb[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                kb[k] = sort_key_of_rank(it[c * 8 + k] >> 16);
+            store_half8(keys, first + c * 8, size, kb);
+        }
+    }
+    if (IDENTITY) {
+        if (active) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                int vb[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    vb[k] = static_cast<int>(it[c * 8 + k] & 0xFFFFu);
+                store_int8(values, first + c * 8, size, vb);
+            }
+        }
+        __syncthreads();
+        return;
+    }
+    // payloads: stage the input values in LDS (every thread has read its items back), gather by position
+    __syncthreads();
+    if (active) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            int vb[8];
+            load_int8(vb, values, first + c * 8, size);
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                buf.item[sort_slot(first + c * 8 + k)] = static_cast<uint32_t>(vb[k]);
+        }
+    }
+    __syncthreads();
+    if (active) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            int vb[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k)
+                vb[k] = static_cast<int>(buf.item[sort_slot(static_cast<int>(it[c * 8 + k] & 0xFFFFu))]);
+            store_int8(values, first + c * 8, size, vb);
+        }
+    }
+    __syncthreads(); // the sorted arrays are visible to the whole workgroup
+}
+
 // ---- cumulative_sum (native/cumulative_sum_kernel.cu:8-26) ---------------------------
 // Inclusive prefix sums in fp32, each rounded to fp16, in place.  A thread sums
 // its 8*CH consecutive values in order, the thread totals are scanned in thread
@@ -390,18 +553,47 @@ __host__ __device__ inline float sampler_coin(unsigned long long seed, int pos)
 }
 
 // Sampler.Sample's stochastic branch (src/Sampler.cs:48-67) on one workgroup.
+// LDS_SORT: size <= kSortLdsItems and `buf` is there; otherwise the sort runs
+// through the second global buffer (keys2, values2).
+// Each phase is a call, not inlined: inlined together the phases' register arrays
+// overlap in the allocator's view and two hundred registers spill.
 template <int CH>
-__device__ __forceinline__ int sample_dev(uint16_t* logits, int* indices, int size, float temperature, float top_p,
-                                          float coin, uint16_t* keys2, int* values2, SamplerLds& lds)
+__device__ __noinline__ void softmax_logits_call(uint16_t* logits, int size, float temperature, int* indices,
+                                                 SamplerLds* lds)
 {
-    softmax_logits_dev<CH>(logits, size, temperature, indices, lds);
+    softmax_logits_dev<CH>(logits, size, temperature, indices, *lds);
+}
+__device__ __noinline__ void sort_lds_identity_call(uint16_t* keys, int* values, int size, SamplerLds* lds, SortLds* buf)
+{
+    sort_lds_dev<true>(keys, values, size, *lds, *buf);
+}
+template <int CH>
+__device__ __noinline__ void sort_call(uint16_t* keys, int* values, int size, uint16_t* keys2, int* values2,
+                                       SamplerLds* lds)
+{
+    sort_dev<CH>(keys, values, size, keys2, values2, *lds);
+}
+template <int CH>
+__device__ __noinline__ void cumulative_sum_call(uint16_t* values, int size, SamplerLds* lds)
+{
+    cumulative_sum_dev<CH>(values, size, *lds);
+}
+
+template <int CH, bool LDS_SORT>
+__device__ __forceinline__ int sample_dev(uint16_t* logits, int* indices, int size, float temperature, float top_p,
+                                          float coin, uint16_t* keys2, int* values2, SamplerLds& lds, SortLds* buf)
+{
+    softmax_logits_call<CH>(logits, size, temperature, indices, &lds);
     __syncthreads();
     float threshold = coin;
     if (!(top_p <= 0.0f || top_p >= 1.0f)) {
-        sort_dev<CH>(logits, indices, size, keys2, values2, lds);
+        if (LDS_SORT)
+            sort_lds_identity_call(logits, indices, size, &lds, buf); // indices are 0..size-1 here
+        else
+            sort_call<CH>(logits, indices, size, keys2, values2, &lds);
         threshold = coin * top_p;
     }
-    cumulative_sum_dev<CH>(logits, size, lds);
+    cumulative_sum_call<CH>(logits, size, &lds);
     __syncthreads();
     return sample_top_p_dev<CH>(logits, indices, size, threshold, lds);
 }
