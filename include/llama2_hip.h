@@ -261,6 +261,29 @@ int llama2_sample_top_p(const llama2_half* logits, const int* indices, int size,
 int llama2_sample(llama2_half* logits, int* indices, int size, float temperature, float top_p,
                   float coin, int* result, int pos);
 
+/* ------------------------------------------------------- converter repack
+ * The tensor transformations of ModelConverter.RepackQWeightByName
+ * (src/ModelConverter.cs:196-275) on device buffers: what turns an AWQ
+ * checkpoint's tensors into the layout every entry point above reads.  All
+ * asynchronous on the library's stream; out and in must not overlap. */
+
+/* RepackQData (src/ModelConverter.cs:277-317).  in: [height][width/8] words of
+ * the AWQ "GEMM" format (nibble i of a word = column 8c + {0,2,4,6,1,3,5,7}[i]);
+ * out: [width][ceil(height/8)] words, word y/8 of row x = rows y..y+7 of column
+ * x.  Used for qweight (height = K) and qzeros (height = K/128).  When height
+ * is not a multiple of 8 the unused nibbles of a row's last word are filled as
+ * the reference fills them (first rows of the next column, zero behind the
+ * last column), so converted files are byte-identical.  width % 8 == 0. */
+int llama2_repack_qdata(uint32_t* out, const uint32_t* in, int height, int width);
+
+/* RepackScales (src/ModelConverter.cs:319-328): [meta_height][width] halfs ->
+ * [width][meta_height]. */
+int llama2_repack_scales(llama2_half* out, const llama2_half* in, int meta_height, int width);
+
+/* The Format.v1 branch (src/ModelConverter.cs:247-262): scale rows stored with
+ * ceil(scales_size/8)*8 halfs each -> rows of scales_size halfs. */
+int llama2_compact_scales_v1(llama2_half* out, const llama2_half* in, int scales_size, int width);
+
 /* ------------------------------------------------------------ decode step */
 
 /* src/Config.cs:6-19 -- the 32-byte model-file header, same field order. */

@@ -102,6 +102,9 @@ _SIGNATURES = {
     "llama2_cumulative_sum": [vp, i],
     "llama2_sample_top_p": [vp, vp, i, f, vp, i],
     "llama2_sample": [vp, vp, i, f, f, f, vp, i],
+    "llama2_repack_qdata": [vp, vp, i, i],
+    "llama2_repack_scales": [vp, vp, i, i],
+    "llama2_compact_scales_v1": [vp, vp, i, i],
     "llama2_decode_create": [C.POINTER(vp), C.POINTER(Config), C.POINTER(TransformerWeights),
                              C.POINTER(RunState), i],
     "llama2_decode_forward": [vp, i, i],

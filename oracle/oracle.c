@@ -52,6 +52,12 @@
  *   sample_top_p .......... brute force over all thresholds on small inputs
  *   sample ................ composition, checked against the empirical
  *                           distribution for a 4-token vocabulary
+ *   repack_qdata .......... an integer matrix packed the way AWQ's GEMM
+ *                           packer is published (column 8c+orderMap[i] in
+ *                           nibble i), repacked, then unpacked by the
+ *                           golden-pinned unpack: the matrix comes back; the
+ *                           spill-over nibbles of ragged heights by brute force
+ *   repack_scales ......... numpy transpose
  *   forward ............... composition checked module by module
  * Parity unpinned: the fp32 summation ORDER of the reference's CUB
  * warp/block reductions (it only matters below fp16 rounding and the
@@ -641,6 +647,67 @@ ORACLE_API float oracle_coin(uint64_t seed, int pos)
     z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
     z ^= z >> 31;
     return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+/* ================================================================== */
+/* Converter repack (the data format on the other side of the loader):   */
+/* src/ModelConverter.cs:196-328.                                        */
+/* ================================================================== */
+
+/* RepackQData, src/ModelConverter.cs:277-317, line for line.  `in` is    */
+/* the AWQ "GEMM" tensor [height][width/8] of uint32: nibble i of a word  */
+/* holds column 8*(word index) + orderMap[i] (orderMap :19).  `out` is    */
+/* [width][ceil(height/8)]: word y/8 of row x holds rows y..y+7 of column */
+/* x.  When height is not a multiple of 8 (the zero points: height =      */
+/* number of groups) the last word of a row picks up the first elements   */
+/* of the NEXT column from the intermediate array (zero behind the last   */
+/* column): those nibbles are don't-care for the kernels but they are     */
+/* part of the file the reference writes, so they are reproduced.         */
+ORACLE_API void ref_repack_qdata(const uint32_t* q_weight_in, int height, int width, uint32_t* q_weight_out)
+{
+    static const int orderMap[8] = {0, 2, 4, 6, 1, 3, 5, 7};
+    uint32_t* packed = (uint32_t*)calloc((size_t)width * height + 8, sizeof(uint32_t));
+    uint32_t q[8];
+    for (int y = 0; y < height; ++y)
+        for (int x = 0; x < width; x += 8) {
+            size_t offset = (size_t)height * x + y;
+            uint32_t packed_q_wt = q_weight_in[((size_t)y * width + x) / 8];
+            for (int i = 0; i < 8; ++i) {
+                q[orderMap[i]] = packed_q_wt & 0xF;
+                packed_q_wt >>= 4;
+            }
+            for (int i = 0; i < 8; ++i)
+                packed[offset + (size_t)height * i] = q[i];
+        }
+    int packed_wt_height = ceil_div(height, 8);
+    for (int x = 0; x < width; ++x)
+        for (int y = 0; y < height; y += 8) {
+            size_t offset = (size_t)height * x + y;
+            uint32_t packed_val = 0;
+            for (int i = 0; i < 8; ++i)
+                packed_val |= packed[offset + i] << (4 * i);
+            q_weight_out[(size_t)x * packed_wt_height + y / 8] = packed_val;
+        }
+    free(packed);
+}
+
+/* RepackScales, src/ModelConverter.cs:319-328: [meta_height][width] ->   */
+/* [width][meta_height].                                                  */
+ORACLE_API void ref_repack_scales(const uint16_t* scales_in, int meta_height, int width, uint16_t* packed)
+{
+    for (int x = 0; x < width; ++x)
+        for (int y = 0; y < meta_height; ++y)
+            packed[(size_t)x * meta_height + y] = scales_in[(size_t)y * width + x];
+}
+
+/* Format.v1 scales, src/ModelConverter.cs:247-262: rows of               */
+/* zeros_size*8 halfs compacted to rows of scales_size halfs.             */
+ORACLE_API void ref_compact_scales_v1(const uint16_t* scales, int scales_size, int width, uint16_t* scales_t)
+{
+    int original_height = ceil_div(scales_size, 8) * 8;
+    for (int x = 0; x < width; ++x)
+        for (int y = 0; y < scales_size; ++y)
+            scales_t[(size_t)x * scales_size + y] = scales[(size_t)x * original_height + y];
 }
 
 /* ================================================================== */

@@ -265,6 +265,30 @@ def f64_cumulative_sum(values):
     return out
 
 
+# ---- converter repack (src/ModelConverter.cs:196-328) -----------------------------------
+def ref_repack_qdata(q_in, height, width):
+    """[height][width/8] AWQ GEMM words -> [width][ceil(height/8)] words."""
+    q_in = np.ascontiguousarray(q_in, np.uint32).ravel()
+    assert q_in.size == height * width // 8 and width % 8 == 0
+    out = np.zeros(width * ((height + 7) // 8), np.uint32)
+    lib().ref_repack_qdata(_u(q_in), C.c_int(height), C.c_int(width), _u(out))
+    return out
+
+
+def ref_repack_scales(scales_in, meta_height, width):
+    scales_in = np.ascontiguousarray(scales_in, np.float16).ravel()
+    out = np.empty(meta_height * width, np.float16)
+    lib().ref_repack_scales(_h(scales_in), C.c_int(meta_height), C.c_int(width), _h(out))
+    return out
+
+
+def ref_compact_scales_v1(scales, scales_size, width):
+    scales = np.ascontiguousarray(scales, np.float16).ravel()
+    out = np.empty(scales_size * width, np.float16)
+    lib().ref_compact_scales_v1(_h(scales), C.c_int(scales_size), C.c_int(width), _h(out))
+    return out
+
+
 # ---- fp64 closed forms ------------------------------------------------------------
 def f64_matvec_int4(x, W, Z, S, K, N):
     y = np.empty(N, np.float64)
