@@ -58,14 +58,14 @@ def main():
     ap.add_argument("--steps", type=int, default=3200)
     ap.add_argument("--warmup", type=int, default=320)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
-    ap.add_argument("--only", default="", help="comma list of legs: set,kernel,calib,attn,decode,sampler,cpu (default: all but calib)")
+    ap.add_argument("--only", default="", help="comma list of legs: set,kernel,calib,attn,decode,sampler,repack,cpu (default: all but calib)")
     ap.add_argument("--decode-mode", default="fused_graph", choices=["modules", "fused", "fused_graph"])
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (batch-1 decode has no cross-GPU exchange to measure); "
             "--gpus %d is not supported" % args.gpus)
         sys.exit(2)
-    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "attn", "decode", "sampler", "cpu"}
+    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "attn", "decode", "sampler", "repack", "cpu"}
 
     from managedllama2_amd import capi, synth
     from managedllama2_amd.device import DeviceVariable, init
@@ -347,6 +347,29 @@ def main():
             (sampler["softmax_logits_us"], sampler["sort_us"], sampler["cumulative_sum_us"],
              sampler["sample_top_p_us"], sampler["four_modules_us"], sampler["one_launch_us"],
              sampler["decode_tokens_per_s"]))
+
+    if "repack" in legs:
+        # the converter's repack of the 7B weight tensors (AWQ GEMM words -> output-major words):
+        # every word read once and written once
+        repack = {}
+        for name, (K, N) in (("qkvo_4096x4096", (dim, dim)), ("gate_up_4096x11008", (dim, hidden)),
+                             ("down_11008x4096", (hidden, dim))):
+            words = K * N // 8
+            src_w = DeviceVariable.from_host(synth.rng_for(8, K, N).integers(0, 2 ** 32, words, dtype=np.uint64)
+                                             .astype(np.uint32))
+            dst_w = DeviceVariable(np.uint32, words)
+            capi.call("llama2_repack_qdata", dst_w.ptr, src_w.ptr, K, N)
+            capi.call("llama2_sync")
+            ev.start()
+            for _ in range(20):
+                capi.call("llama2_repack_qdata", dst_w.ptr, src_w.ptr, K, N)
+            us = 1e3 * ev.stop_ms() / 20
+            repack[name] = {"us": round(us, 2), "GBps_read_plus_write": round(2 * words * 4 / us / 1e3, 1)}
+            src_w.free()
+            dst_w.free()
+        result["repack"] = repack
+        log("repack (read+write): " + ", ".join("%s %.1f us %.0f GB/s" % (k, v["us"], v["GBps_read_plus_write"])
+                                                for k, v in repack.items()))
 
     if "cpu" in legs and args.cpu_seconds > 0:
         from oracle import oracle

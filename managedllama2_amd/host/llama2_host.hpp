@@ -492,6 +492,47 @@ class Sampler {
     Sort sort_;
 };
 
+// ---------------------------------------------------------------- src/ModelConverter.cs:196-328 (tensor side)
+// RepackQWeightByName on host arrays: upload, repack on the GPU, download.  Reading the PyTorch
+// checkpoint (zip + pickle) is outside this path; the caller brings the three tensors.
+struct ModelConverter {
+    enum class Format { v0, v1 };
+    struct Repacked {
+        std::vector<uint32_t> Weight, Zeros;
+        std::vector<Half> Scales;
+    };
+    static int CeilDiv(int a, int b) { return (a + (b - 1)) / b; }
+    static Repacked RepackQWeight(const uint32_t* qweight, const uint32_t* qzeros, const Half* scales, int height,
+                                  int width, Format format)
+    {
+        const int groupSize = 128;
+        const int scalesSize = CeilDiv(height, groupSize), weightsSize = CeilDiv(height, 8),
+                  zerosSize = CeilDiv(scalesSize, 8);
+        Repacked r;
+        if (format == Format::v0) {
+            const size_t w8 = static_cast<size_t>(CeilDiv(width, 8));
+            DeviceVariable<uint32_t> wIn(qweight, w8 * height), wOut(static_cast<size_t>(weightsSize) * width);
+            Check(llama2_repack_qdata(wOut.DevicePointer(), wIn.DevicePointer(), height, width)); // :238
+            DeviceVariable<uint32_t> zIn(qzeros, w8 * scalesSize), zOut(static_cast<size_t>(zerosSize) * width);
+            Check(llama2_repack_qdata(zOut.DevicePointer(), zIn.DevicePointer(), scalesSize, width)); // :239
+            DeviceVariable<Half> sIn(scales, static_cast<size_t>(scalesSize) * width),
+                sOut(static_cast<size_t>(scalesSize) * width);
+            Check(llama2_repack_scales(sOut.DevicePointer(), sIn.DevicePointer(), scalesSize, width)); // :240
+            r.Weight = wOut.ToHost();
+            r.Zeros = zOut.ToHost();
+            r.Scales = sOut.ToHost();
+        } else {
+            r.Weight.assign(qweight, qweight + static_cast<size_t>(weightsSize) * width);
+            r.Zeros.assign(qzeros, qzeros + static_cast<size_t>(zerosSize) * width);
+            DeviceVariable<Half> sIn(scales, static_cast<size_t>(zerosSize) * 8 * width),
+                sOut(static_cast<size_t>(scalesSize) * width);
+            Check(llama2_compact_scales_v1(sOut.DevicePointer(), sIn.DevicePointer(), scalesSize, width)); // :247-262
+            r.Scales = sOut.ToHost();
+        }
+        return r;
+    }
+};
+
 // ---------------------------------------------------------------- src/ITransformer.cs, src/Transformer.cs
 struct ITransformer {
     virtual ~ITransformer() = default;

@@ -3,6 +3,7 @@
 // reference's ITransformer.  Builds into libllama2_host.so.
 #include "llama2_host.hpp"
 
+#include <algorithm>
 #include <string>
 
 using namespace libLlama2;
@@ -50,6 +51,21 @@ __attribute__((visibility("default"))) int l2h_check_model_file(const char* path
         if (TransformerWeights::ExpectedBytes(c) != remaining)
             throw FileLoadException("Failed to read file. offset: " + std::to_string(TransformerWeights::ExpectedBytes(c)) +
                                     " != length: " + std::to_string(remaining));
+    });
+}
+
+// ModelConverter::RepackQWeight on caller-provided host arrays; out_* sized as in the model file.
+__attribute__((visibility("default"))) int l2h_repack_qweight(const uint32_t* qweight, const uint32_t* qzeros,
+                                                              const uint16_t* scales, int height, int width, int format,
+                                                              uint32_t* out_weight, uint32_t* out_zeros, uint16_t* out_scales)
+{
+    return guarded([&] {
+        Check(llama2_init(0));
+        auto r = ModelConverter::RepackQWeight(qweight, qzeros, scales, height, width,
+                                               format == 0 ? ModelConverter::Format::v0 : ModelConverter::Format::v1);
+        std::copy(r.Weight.begin(), r.Weight.end(), out_weight);
+        std::copy(r.Zeros.begin(), r.Zeros.end(), out_zeros);
+        std::copy(r.Scales.begin(), r.Scales.end(), out_scales);
     });
 }
 

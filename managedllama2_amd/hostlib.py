@@ -29,6 +29,8 @@ def load():
         lib.l2h_transformer_open.argtypes = [C.c_char_p, C.c_int, C.c_int, C.POINTER(C.c_void_p)]
         lib.l2h_transformer_open_sampled.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_float, C.c_float,
                                                      C.c_ulonglong, C.POINTER(C.c_void_p)]
+        u32p, u16p = C.POINTER(C.c_uint32), C.POINTER(C.c_uint16)
+        lib.l2h_repack_qweight.argtypes = [u32p, u32p, u16p, C.c_int, C.c_int, C.c_int, u32p, u32p, u16p]
         lib.l2h_transformer_generate.argtypes = [C.c_void_p, C.POINTER(C.c_int), C.c_int, C.c_int, C.POINTER(C.c_int),
                                                  C.POINTER(C.c_int)]
         lib.l2h_transformer_logits.argtypes = [C.c_void_p, C.POINTER(C.c_uint16), C.c_int]
@@ -79,3 +81,19 @@ class Transformer:
         if self._h:
             _check(load().l2h_transformer_close(self._h))
             self._h = C.c_void_p()
+
+
+def repack_qweight(qweight, qzeros, scales, height, width, fmt=0):
+    """libLlama2::ModelConverter::RepackQWeight (fmt 0 = Format.v0, 1 = Format.v1) -> (Weight, Zeros, Scales)."""
+    ss = (height + 127) // 128
+    W = np.empty(((height + 7) // 8) * width, np.uint32)
+    Z = np.empty(((ss + 7) // 8) * width, np.uint32)
+    S = np.empty(ss * width, np.float16)
+    qweight = np.ascontiguousarray(qweight, np.uint32).ravel()
+    qzeros = np.ascontiguousarray(qzeros, np.uint32).ravel()
+    scales = np.ascontiguousarray(scales, np.float16).ravel()
+    u32p, u16p = C.POINTER(C.c_uint32), C.POINTER(C.c_uint16)
+    _check(load().l2h_repack_qweight(qweight.ctypes.data_as(u32p), qzeros.ctypes.data_as(u32p),
+                                     scales.ctypes.data_as(u16p), height, width, fmt, W.ctypes.data_as(u32p),
+                                     Z.ctypes.data_as(u32p), S.ctypes.data_as(u16p)))
+    return W, Z, S

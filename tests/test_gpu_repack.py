@@ -7,7 +7,7 @@ decode equals that of the model built directly in the target layout."""
 import numpy as np
 import pytest
 
-from managedllama2_amd import capi, modelconvert, modelfile, synth
+from managedllama2_amd import capi, hostlib, modelconvert, modelfile, synth
 from managedllama2_amd.transformer import Transformer
 from gpu_util import up
 
@@ -138,3 +138,15 @@ def test_v1_format(oracle):
     padded[:, :ss] = S.reshape(N, ss)
     W2, Z2, S2 = modelconvert.RepackQWeight(W, Z, padded, K, N, modelconvert.V1)
     assert np.array_equal(W2, W) and np.array_equal(Z2, Z) and np.array_equal(S2.view(np.uint16), S.view(np.uint16))
+
+
+def test_cpp_host_repack_equals_python(oracle):
+    rng = synth.rng_for(1106)
+    K, N = 11008, 128
+    G = K // 128
+    qw, qz = awq_pack(rng.integers(0, 16, (K, N))), awq_pack(rng.integers(0, 16, (G, N)))
+    sc = (0.002 + 0.018 * rng.random((G, N))).astype(np.float16)
+    W, Z, S = hostlib.repack_qweight(qw, qz, sc, K, N)
+    assert np.array_equal(W, oracle.ref_repack_qdata(qw, K, N))
+    assert np.array_equal(Z, oracle.ref_repack_qdata(qz, G, N))
+    assert np.array_equal(S.view(np.uint16), oracle.ref_repack_scales(sc, G, N).view(np.uint16))
