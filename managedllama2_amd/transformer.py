@@ -8,7 +8,7 @@ import math
 import numpy as np
 
 from . import capi
-from .device import DeviceVariable, QWeight, init
+from .device import DeviceArena, DeviceVariable, QWeight, init
 from .modules import (Argmax, CumulativeSum, Embedding, MatVec, MatVecResidual, MatVecStrided, MatVecSwiGLU,
                       QKVMatVec, RMSNorm, RoPERotation, SampleTopP, Softmax, SoftmaxLogits, Sort, VecMat)
 
@@ -29,20 +29,28 @@ class TransformerWeights:
 
     def __init__(self, config, host):
         self.config = config
-        up = DeviceVariable.from_host
+        from . import modelfile
+        cfg = {k: getattr(config, k) for k in modelfile.FIELDS}
+        tensors = 3 + config.n_layers * (7 * 3 + 2)
+        self.arena = DeviceArena(modelfile.expected_size(cfg) + tensors * DeviceArena.ALIGN)
+        up = self.arena.from_host
+
+        def upq(W, Z, S):
+            return QWeight(up(W), up(Z), up(S))
+
         self.tokenEmbeddingTable = up(host["embedding"])
         self.classifierWeights = up(host["classifier"])
         self.rmsFinalWeight = up(host["rms_final"])
         self.layers = []
         for L in host["layers"]:
             w = PerLayerWeight()
-            w.queryWeight = QWeight.from_host(*L["q"])
-            w.keyWeight = QWeight.from_host(*L["k"])
-            w.valueWeight = QWeight.from_host(*L["v"])
-            w.outputWeight = QWeight.from_host(*L["o"])
-            w.upWeight = QWeight.from_host(*L["up"])
-            w.gateWeight = QWeight.from_host(*L["gate"])
-            w.downWeight = QWeight.from_host(*L["down"])
+            w.queryWeight = upq(*L["q"])
+            w.keyWeight = upq(*L["k"])
+            w.valueWeight = upq(*L["v"])
+            w.outputWeight = upq(*L["o"])
+            w.upWeight = upq(*L["up"])
+            w.gateWeight = upq(*L["gate"])
+            w.downWeight = upq(*L["down"])
             w.rmsAttentionWeight = up(L["rms_att"])
             w.rmsFeedForwardWeight = up(L["rms_ffn"])
             self.layers.append(w)
