@@ -28,6 +28,10 @@ import numpy as np
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the dominant kernel (fused SwiGLU, 46 880 256 algorithmic bytes), measured with
+# two rocprofv3 --pmc runs of `bench.py --only kernel,calib` (counters cannot be read from inside this
+# process): (FETCH_SIZE 23111.6 KiB x 2.000 + WRITE_SIZE 86.0 KiB x 1.000) x 1024
+SWIGLU_HBM_TRAFFIC_BYTES = 47420417
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
 
@@ -202,7 +206,10 @@ def main():
         dom = per_kernel["swiglu"]
         result["roofline"] = {"bound": "hbm", "kernel": "int4_matvec_kernel<2, SWIGLU> (fused gate/up, 2x11008x4096)",
                               "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                              "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                              "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": SWIGLU_HBM_TRAFFIC_BYTES,
+                              "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a "
+                                                "1 GiB copy kernel (factors 2.000 / 1.000): profiles/"
+                                                "int4_matvec_7b_layer_set_hbm_traffic.md",
                               "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_us": dom["us"]}
         result["per_kernel"] = per_kernel
 
