@@ -183,7 +183,6 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     __shared__ float rope_tab[MODE == QKV_ROPE ? kRopeHeadSize : 2]; // (cos, sin) pairs
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int total_waves = gridDim.x * WAVES;
-    const int pos = (MODE == QKV_ROPE || STAGE == STAGE_RMSNORM) && a.pos_ptr ? a.pos_ptr[0] : 0;
     const int pairs = a.N >> 1; // QKV_ROPE: (i, i+64) row pairs per tensor
     const int nitems = MODE == QKV_ROPE ? 3 * pairs : a.n_tensors * a.N;
     int item = blockIdx.x * WAVES + wave;
@@ -211,7 +210,7 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     VecPieces<J> xp;
     const uint16_t* xsrc = a.x;
     if (STAGE == STAGE_RMSNORM && a.embedding) { // native/embedding_kernel.cu:9-11
-        int token = a.tokens[pos];
+        int token = a.tokens[a.pos_ptr ? a.pos_ptr[0] : 0];
         token = token < 0 ? 0 : (token >= a.vocab ? a.vocab - 1 : token); // never read outside the table
         xsrc = a.embedding + static_cast<size_t>(token) * a.K;
     }
@@ -224,6 +223,9 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     if (item < nitems)
         load_item(cur, cur_res, item);
 
+    // The position lives in device memory: outside layer 0 it is read only here, after the weight
+    // loads above were issued.
+    const int pos = MODE == QKV_ROPE && a.pos_ptr ? a.pos_ptr[0] : 0;
     if (MODE == QKV_ROPE) {
         if (a.rope_table) { // prepared by the kernel that set the position
             if (threadIdx.x < kRopeHeadSize)
