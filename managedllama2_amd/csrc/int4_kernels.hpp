@@ -174,7 +174,7 @@ __device__ __forceinline__ void rope_cos_sin(float& fcr, float& fci, int i, int 
 template <int J, int MODE, int STAGE>
 __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
 {
-    constexpr int R = (MODE == SWIGLU || MODE == QKV_ROPE) ? 2 : 1;
+    constexpr int R = MODE == SWIGLU ? 2 : 1;
     constexpr int JC = J * 64;
     constexpr int WAVES = 4;
     __shared__ u32x4 xs[4 * JC];
@@ -186,18 +186,20 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     const int pairs = a.N >> 1; // QKV_ROPE: (i, i+64) row pairs per tensor
     const int nitems = MODE == QKV_ROPE ? 3 * pairs : a.n_tensors * a.N;
     int item = blockIdx.x * WAVES + wave;
+    // QKV_ROPE: an item is a pair of rows (i, i + 64) of one head; a wavefront takes the two rows one
+    // after the other (half 0, half 1) and rotates them when the second is done.
+    int half = 0;
 
-    auto load_item = [&](Frag<J, R>& f, uint16_t& res, int it) {
+    auto load_item = [&](Frag<J, R>& f, uint16_t& res, int it, int hf) {
         it = __builtin_amdgcn_readfirstlane(it);
+        hf = __builtin_amdgcn_readfirstlane(hf);
         if (MODE == SWIGLU) {
             load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[0], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
             load_row<J>(f.w[R - 1], f.zw[R - 1], f.sb[R - 1], a.m[1], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
         } else if (MODE == QKV_ROPE) {
             const int t = (it >= pairs) + (it >= 2 * pairs), rem = it - t * pairs;
             const int n0 = (rem >> 6) * kRopeHeadSize + (rem & 63);
-            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[t], static_cast<size_t>(n0), a.ws, a.ss, a.zs, lane);
-            load_row<J>(f.w[R - 1], f.zw[R - 1], f.sb[R - 1], a.m[t], static_cast<size_t>(n0 + 64), a.ws, a.ss, a.zs,
-                        lane);
+            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[t], static_cast<size_t>(n0 + 64 * hf), a.ws, a.ss, a.zs, lane);
         } else {
             const int t = (it >= a.N) + (it >= 2 * a.N), n = it - t * a.N; // at most 3 tensors
             load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[t], static_cast<size_t>(n), a.ws, a.ss, a.zs, lane);
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     Frag<J, R> cur;
     uint16_t cur_res = 0;
     if (item < nitems)
-        load_item(cur, cur_res, item);
+        load_item(cur, cur_res, item, 0);
 
     // The position lives in device memory: outside layer 0 it is read only here, after the weight
     // loads above were issued.
@@ -252,11 +254,14 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     __syncthreads();
 
     const int zshift = ((lane >> 2) & 7) * 4; // nibble of the zero word: group (c/4) % 8, same for every j
-    for (; item < nitems; item += total_waves) {
+    float v_first = 0.0f;
+    while (item < nitems) {
+        const int nitem = (MODE != QKV_ROPE || half) ? item + total_waves : item;
+        const int nhalf = MODE == QKV_ROPE ? half ^ 1 : 0;
         Frag<J, R> nxt;
         uint16_t nxt_res = 0;
-        if (item + total_waves < nitems)
-            load_item(nxt, nxt_res, item + total_waves);
+        if (nitem < nitems)
+            load_item(nxt, nxt_res, nitem, nhalf);
         float acc[R];
         dot_frag<J, R>(acc, cur, xs, sx, lane, zshift);
         if (MODE == SWIGLU) {
@@ -270,9 +275,11 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
             }
         } else if (MODE == QKV_ROPE) {
             // the unfused path stores q/k as fp16 and RoPE reads them back: keep that rounding
-            const float v0 = half_bits_to_float(float_to_half_bits(wave_sum(acc[0])));
-            const float v1 = half_bits_to_float(float_to_half_bits(wave_sum(acc[R - 1])));
-            if (lane == 0) {
+            const float v = half_bits_to_float(float_to_half_bits(wave_sum(acc[0])));
+            if (half == 0)
+                v_first = v;
+            const float v0 = v_first, v1 = v;
+            if (half == 1 && lane == 0) {
                 const int t = (item >= pairs) + (item >= 2 * pairs), rem = item - t * pairs;
                 const int i = rem & 63, n0 = (rem >> 6) * kRopeHeadSize + i;
                 uint16_t* dst = t == 0 ? a.out[0] : a.out[t] + static_cast<size_t>(pos) * a.kv_dim;
@@ -296,6 +303,8 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
         }
         cur = nxt;
         cur_res = nxt_res;
+        item = nitem;
+        half = nhalf;
     }
 }
 
