@@ -174,7 +174,11 @@ __device__ __forceinline__ void rope_cos_sin(float& fcr, float& fci, int i, int 
 template <int J, int MODE, int STAGE>
 __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
 {
-    constexpr int R = MODE == SWIGLU ? 2 : 1;
+    // Two rows per item (QKV_ROPE: rows i and i + 64 of a head; SWIGLU: gate row and up row) are taken
+    // one after the other by the same wavefront (PAIRED), except where the input is normalised while it
+    // is staged: there holding both rows of SwiGLU at once (R = 2) measured faster.
+    constexpr bool PAIRED = MODE == QKV_ROPE || (MODE == SWIGLU && STAGE == STAGE_X);
+    constexpr int R = (MODE == SWIGLU && !PAIRED) ? 2 : 1;
     constexpr int JC = J * 64;
     constexpr int WAVES = 4;
     __shared__ u32x4 xs[4 * JC];
@@ -186,14 +190,14 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     const int pairs = a.N >> 1; // QKV_ROPE: (i, i+64) row pairs per tensor
     const int nitems = MODE == QKV_ROPE ? 3 * pairs : a.n_tensors * a.N;
     int item = blockIdx.x * WAVES + wave;
-    // QKV_ROPE: an item is a pair of rows (i, i + 64) of one head; a wavefront takes the two rows one
-    // after the other (half 0, half 1) and rotates them when the second is done.
-    int half = 0;
+    int half = 0; // PAIRED: which row of the item's pair is being worked on
 
     auto load_item = [&](Frag<J, R>& f, uint16_t& res, int it, int hf) {
         it = __builtin_amdgcn_readfirstlane(it);
         hf = __builtin_amdgcn_readfirstlane(hf);
-        if (MODE == SWIGLU) {
+        if (MODE == SWIGLU && PAIRED) { // half 0: gate row, half 1: up row
+            load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[hf], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
+        } else if (MODE == SWIGLU) {
             load_row<J>(f.w[0], f.zw[0], f.sb[0], a.m[0], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
             load_row<J>(f.w[R - 1], f.zw[R - 1], f.sb[R - 1], a.m[1], static_cast<size_t>(it), a.ws, a.ss, a.zs, lane);
         } else if (MODE == QKV_ROPE) {
@@ -256,8 +260,8 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     const int zshift = ((lane >> 2) & 7) * 4; // nibble of the zero word: group (c/4) % 8, same for every j
     float v_first = 0.0f;
     while (item < nitems) {
-        const int nitem = (MODE != QKV_ROPE || half) ? item + total_waves : item;
-        const int nhalf = MODE == QKV_ROPE ? half ^ 1 : 0;
+        const int nitem = (!PAIRED || half) ? item + total_waves : item;
+        const int nhalf = PAIRED ? half ^ 1 : 0;
         Frag<J, R> nxt;
         uint16_t nxt_res = 0;
         if (nitem < nitems)
@@ -265,9 +269,16 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
         float acc[R];
         dot_frag<J, R>(acc, cur, xs, sx, lane, zshift);
         if (MODE == SWIGLU) {
-            const float g = wave_sum(acc[0]);
-            const float u = wave_sum(acc[R - 1]);
-            if (lane == 0) {
+            float g = wave_sum(acc[0]), u = 0.0f;
+            if (PAIRED) {
+                if (half == 0)
+                    v_first = g;
+                u = g;
+                g = v_first;
+            } else {
+                u = wave_sum(acc[R - 1]);
+            }
+            if ((!PAIRED || half == 1) && lane == 0) {
                 float v = g;
                 v *= 1.0f / (1.0f + expf(-v)); // native/mat_vec_kernel.cu:219-221
                 v *= u;
