@@ -30,8 +30,8 @@ sys.path.insert(0, ROOT)
 
 # HBM bytes per launch of the dominant kernel (fused SwiGLU, 46 880 256 algorithmic bytes), measured with
 # two rocprofv3 --pmc runs of `bench.py --only kernel,calib` (counters cannot be read from inside this
-# process): (FETCH_SIZE 23111.6 KiB x 2.000 + WRITE_SIZE 86.0 KiB x 1.000) x 1024
-SWIGLU_HBM_TRAFFIC_BYTES = 47420417
+# process): (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000) x 1024
+SWIGLU_HBM_TRAFFIC_BYTES = 47409114
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
 
