@@ -207,6 +207,16 @@ def test_llama7b_shaped_layers(oracle, mode):
     assert exact >= len(gen) - 1
 
 
+@pytest.mark.parametrize("mode", [capi.DECODE_MODULES, capi.DECODE_FUSED | capi.DECODE_GRAPH])
+def test_llama13b_shaped_layers(oracle, mode):
+    """Real 13B tensor shapes (dim 5120, hidden 13824, 40 heads): 3 and 7 chunk columns per lane with a
+    half-filled last column, 14 zero-point words per row of the down projection."""
+    cfg = dict(synth.LLAMA2_13B, n_layers=2, seq_len=32)
+    model = synth.random_model(cfg, seed=12)
+    exact, gen, _ = run_and_check(oracle, cfg, model, mode, n_prompt=3, steps=6, seed=409)
+    assert exact >= len(gen) - 1
+
+
 def test_decoder_rejects_what_the_reference_rejects():
     import ctypes as C
     model = synth.random_model(SMALL, seed=5)
