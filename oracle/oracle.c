@@ -440,6 +440,8 @@ ORACLE_API void ref_vecmat(uint16_t* out, const uint16_t* att, const uint16_t* v
 /* softmax of one row, in place: test/SoftmaxTests.cs:31-59. */
 ORACLE_API void ref_softmax(uint16_t* x1, int size)
 {
+    if (size <= 0)
+        return;
     float* x = (float*)malloc(sizeof(float) * (size_t)size);
     for (int i = 0; i < size; ++i)
         x[i] = h2f(x1[i]);
