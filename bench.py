@@ -183,12 +183,20 @@ def main():
         wall0 = time.perf_counter()
         ms = timed_replays(graph, replays)
         wall = time.perf_counter() - wall0
+        # the spread over replays (one replay = one pass over the 32 layers), each timed on its own
+        per_replay = []
+        for _ in range(min(replays, 50)):
+            ev.start()
+            capi.call("llama2_graph_launch", graph)
+            per_replay.append(ev.stop_ms() / n_layers)
+        q = np.percentile(np.array(per_replay), [10, 50, 90])
         capi.call("llama2_graph_destroy", graph)
         ms_per_step = ms / steps
         gbps = sizes["total"] / (ms_per_step * 1e-3) / 1e9
         result.update(steps=steps, value=round(gbps, 1), ms_per_step=round(ms_per_step, 5),
                       pct_of_hbm_peak=round(100 * gbps / HBM_PEAK_GBPS, 2),
-                      wall_ms_per_step=round(1e3 * wall / steps, 5))
+                      wall_ms_per_step=round(1e3 * wall / steps, 5),
+                      ms_per_step_p10_median_p90=[round(float(v), 5) for v in q])
         log("layer mat-vec set: %.2f us/step, %.0f GB/s (%.1f%% of 8 TB/s)" %
             (1e3 * ms_per_step, gbps, 100 * gbps / HBM_PEAK_GBPS))
 
