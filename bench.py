@@ -310,6 +310,13 @@ def main():
                             "pct_of_hbm_peak": round(100 * bytes_tok * tok_s / 1e9 / HBM_PEAK_GBPS, 2),
                             "bandwidth_bound_tokens_per_s": round(HBM_PEAK_GBPS * 1e9 / bytes_tok, 1),
                             "last_tokens": [int(t) for t in toks[-4:]]}
+        # the reference's own loop shape (Transformer.Generate: forward, sample, read the token back on the
+        # host every step) over the same launches: what a host that keeps its loop gets
+        t1 = time.perf_counter()
+        n_host = sum(1 for _ in model.Generate(prompt, 192, stop_on_special=False))
+        host_tok_s = n_host / (time.perf_counter() - t1)
+        result["decode"]["host_loop_tokens_per_s"] = round(host_tok_s, 1)
+        log("decode, host loop with one read-back per token: %.1f tok/s" % host_tok_s)
         log("decode: %.1f tok/s (%.3f ms/token, %.0f GB/s = %.1f%% of peak; ceiling %.0f tok/s)" %
             (tok_s, ms / steps, bytes_tok * tok_s / 1e9, 100 * bytes_tok * tok_s / 1e9 / HBM_PEAK_GBPS,
              HBM_PEAK_GBPS * 1e9 / bytes_tok))
