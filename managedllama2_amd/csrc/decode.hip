@@ -43,6 +43,7 @@ constexpr int kMaxSplits = 64; // one lane per block in the merge
 constexpr int kPartStride = kRopeHeadSize + 2; // 128 partial outputs, block max, block sum
 
 inline int attn_max_splits(int seq_len) { return ceil_div(seq_len, kSplitT); }
+constexpr int kSmallBlockMaxSeq = 3072; // llama2_multi_head_attention: 128-row blocks up to this length
 
 struct AttnArgs {
     const uint16_t* q;
@@ -607,7 +608,12 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
     L2_CHECK(n_heads <= kMaxAttnHeads, "%s: n_heads=%d exceeds %d", fn, n_heads, kMaxAttnHeads);
     L2_CHECK((static_cast<long long>(seq_length) + kSplitT) * dim * 2 < (1ll << 31),
              "%s: seq_length * dim = %lld is too large", fn, static_cast<long long>(seq_length) * dim);
-    const int splits = attn_max_splits(seq_length);
+    // The caller knows the length here (the decode step does not: its position lives on the device), so
+    // the block can be matched to it: 4-wavefront workgroups over 128-row blocks spread a short
+    // sequence over more compute units, 16-wavefront workgroups over 512-row blocks need fewer merges.
+    const bool small_blocks = seq_length <= kSmallBlockMaxSeq;
+    const int block_t = small_blocks ? 128 : kSplitT;
+    const int splits = ceil_div(seq_length, block_t);
     L2_CHECK(splits <= kMaxSplits, "%s: seq_length=%d exceeds %d", fn, seq_length, kMaxSplits * kSplitT);
     if (splits > 1)
         L2_TRY(ensure_attn_partials(sizeof(float) * static_cast<size_t>(n_heads) * splits * kPartStride));
@@ -615,7 +621,10 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
     a.q = query, a.kcache = key, a.vcache = value, a.out = output;
     a.part = ctx().attn_partials, a.counters = ctx().attn_counters, a.pos_ptr = nullptr, a.seq = seq_length;
     a.dim = dim, a.max_splits = splits, a.scale = scale;
-    hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(splits, n_heads), dim3(kAttnWaves * 64), 0, ctx().stream, a);
+    if (small_blocks)
+        hipLaunchKernelGGL(fused_attn_kernel<4>, dim3(splits, n_heads), dim3(256), 0, ctx().stream, a);
+    else
+        hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(splits, n_heads), dim3(kAttnWaves * 64), 0, ctx().stream, a);
     L2_LAUNCH_CHECK(fn);
     return LLAMA2_OK;
 }
