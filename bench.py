@@ -189,14 +189,14 @@ def main():
             ev.start()
             capi.call("llama2_graph_launch", graph)
             per_replay.append(ev.stop_ms() / n_layers)
-        q = np.percentile(np.array(per_replay), [10, 50, 90])
+        spread = np.percentile(np.array(per_replay), [10, 50, 90])
         capi.call("llama2_graph_destroy", graph)
         ms_per_step = ms / steps
         gbps = sizes["total"] / (ms_per_step * 1e-3) / 1e9
         result.update(steps=steps, value=round(gbps, 1), ms_per_step=round(ms_per_step, 5),
                       pct_of_hbm_peak=round(100 * gbps / HBM_PEAK_GBPS, 2),
                       wall_ms_per_step=round(1e3 * wall / steps, 5),
-                      ms_per_step_p10_median_p90=[round(float(v), 5) for v in q])
+                      ms_per_step_p10_median_p90=[round(float(v), 5) for v in spread])
         log("layer mat-vec set: %.2f us/step, %.0f GB/s (%.1f%% of 8 TB/s)" %
             (1e3 * ms_per_step, gbps, 100 * gbps / HBM_PEAK_GBPS))
 

@@ -23,27 +23,52 @@
 namespace l2 {
 
 // ---------------------------------------------------------------- fused attention
-// One workgroup of 16 wavefronts per (head, block of timesteps).  Every byte of K
-// and V the workgroup needs is requested before the first score is computed (up
-// to 16 loads of 16 bytes per lane; rows outside the block are out of the
+// One workgroup of WAVES wavefronts per (head, block of 32 * WAVES timesteps).  Every
+// byte of K and V the workgroup needs is requested before the first score is computed
+// (up to 16 loads of 16 bytes per lane; rows outside the block are out of the
 // buffer's range and cost no traffic), 16 lanes share one timestep, scores are
 // rounded to fp16 like the reference's `attention` buffer, softmax statistics
 // are per block and the blocks of a head are merged by whichever workgroup
 // finishes last (fixed merge order: deterministic).
 //
-// One compute unit pulls only a few tens of GB/s, the exchange between
-// workgroups costs about 3 us (write-through stores, an atomic, two dependent
-// reads) and dispatching many 1024-thread workgroups that find nothing to do is
-// not free either (blocks of 128 or 256 rows measured slower at every length).
-// So a block is 512 rows: up to that length a head is one workgroup and needs
-// no exchange at all.
+// One compute unit pulls only a few tens of GB/s, so a short sequence wants
+// many small blocks (4 wavefronts, 128 rows); the exchange between workgroups
+// costs about 3 us whatever their number, and a long sequence wants fewer
+// merges (16 wavefronts, 512 rows).  Dispatching workgroups that find nothing
+// to do is not free: a grid sized for the whole context costs several
+// microseconds per launch at short lengths.  The position lives on the device,
+// but the host always knows an upper bound for it, so it picks the launch
+// shape (block size, number of blocks) from a short list by that bound.
 constexpr int kAttnWaves = 16;
 constexpr int kSplitT = 32 * kAttnWaves; // 512
+constexpr int kSmallWaves = 4;
+constexpr int kSmallSplitT = 32 * kSmallWaves; // 128
 constexpr int kMaxSplits = 64; // one lane per block in the merge
 constexpr int kPartStride = kRopeHeadSize + 2; // 128 partial outputs, block max, block sum
 
 inline int attn_max_splits(int seq_len) { return ceil_div(seq_len, kSplitT); }
-constexpr int kSmallBlockMaxSeq = 3072; // llama2_multi_head_attention: 128-row blocks up to this length
+constexpr int kSmallBlockMaxSeq = 3072; // 128-row blocks up to this length, 512-row blocks beyond
+
+// Launch shapes of the decode step: index b < kAttnShapes - 1 is 2^b blocks of 128
+// rows, the last index is 512-row blocks over the whole context.
+constexpr int ceil_log2(int v) { return v <= 1 ? 0 : 1 + ceil_log2((v + 1) / 2); }
+constexpr int kAttnShapes = ceil_log2(kSmallBlockMaxSeq / kSmallSplitT) + 2;
+struct AttnShape {
+    int waves;
+    int splits;
+};
+inline int attn_shape_index(int rows)
+{
+    if (rows > kSmallBlockMaxSeq)
+        return kAttnShapes - 1;
+    return ceil_log2(ceil_div(rows, kSmallSplitT));
+}
+inline AttnShape attn_shape(int index, int seq_len)
+{
+    if (index == kAttnShapes - 1)
+        return AttnShape{kAttnWaves, attn_max_splits(seq_len)};
+    return AttnShape{kSmallWaves, 1 << index};
+}
 
 struct AttnArgs {
     const uint16_t* q;
@@ -375,11 +400,11 @@ struct llama2_decoder {
     int* state = nullptr;
     float* attn_part = nullptr;
     unsigned* counters = nullptr;
-    int max_splits = 0;
-    hipGraphExec_t graph_forward = nullptr; // Transformer.Forward
-    hipGraphExec_t graph_step = nullptr;    // Forward + greedy sample + position advance
-    // Forward + stochastic sample + position advance, captured for the parameters below
-    hipGraphExec_t graph_step_sampled = nullptr;
+    // One captured graph per (kind, attention launch shape).  Kinds: Transformer.Forward;
+    // Forward + greedy sample + position advance; Forward + stochastic sample + position
+    // advance, captured for the parameters below.
+    enum { kGraphForward, kGraphStep, kGraphStepSampled, kGraphKinds };
+    hipGraphExec_t graphs[kGraphKinds][l2::kAttnShapes] = {};
     float sampled_temperature = 0.0f, sampled_top_p = 0.0f;
     unsigned long long sampled_seed = 0;
 };
@@ -445,9 +470,11 @@ int forward_modules(llama2_decoder* d, int position, int next_position)
 
 QW qw(const llama2_qweight& q) { return QW{q.weight, q.zeros, q.scales}; }
 
-// The same step in 5 launches per layer; the position comes from d->state.
-int forward_fused(llama2_decoder* d)
+// The same step in 5 launches per layer; the position comes from d->state, and
+// `shape` (attn_shape_index of an upper bound of position + 1) sizes the attention grid.
+int forward_fused(llama2_decoder* d, int shape)
 {
+    const AttnShape as = attn_shape(shape, d->cfg.seq_len);
     const llama2_config& c = d->cfg;
     const llama2_run_state& s = d->s;
     const int dim = c.dim, hidden = c.hidden_dim;
@@ -474,10 +501,14 @@ int forward_fused(llama2_decoder* d)
             AttnArgs a{}; // :175 (MultiHeadAttention :150-156)
             a.q = s.q, a.kcache = s.key_cache + layer_offset, a.vcache = s.value_cache + layer_offset, a.out = s.xb;
             a.part = d->attn_part, a.counters = d->counters, a.pos_ptr = d->state;
-            a.dim = dim, a.max_splits = d->max_splits;
+            a.dim = dim, a.max_splits = as.splits;
             a.scale = 1.0f / sqrtf(static_cast<float>(d->head_size));
-            hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(d->max_splits, c.n_heads), dim3(kAttnWaves * 64), 0,
-                               ctx().stream, a);
+            if (as.waves == kSmallWaves)
+                hipLaunchKernelGGL(fused_attn_kernel<kSmallWaves>, dim3(as.splits, c.n_heads), dim3(kSmallWaves * 64), 0,
+                                   ctx().stream, a);
+            else
+                hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(as.splits, c.n_heads), dim3(kAttnWaves * 64),
+                                   0, ctx().stream, a);
             L2_LAUNCH_CHECK("fused attention");
         }
         {
@@ -544,14 +575,15 @@ int set_state(llama2_decoder* d, int pos, int n_prompt, int advance)
     return LLAMA2_OK;
 }
 
-int capture(hipGraphExec_t* exec, llama2_decoder* d, bool with_sample, bool stochastic = false)
+int capture(hipGraphExec_t* exec, llama2_decoder* d, int kind, int shape)
 {
     L2_HIP(hipStreamBeginCapture(ctx().stream, hipStreamCaptureModeThreadLocal));
     ctx().capturing = true;
-    int rc = forward_fused(d);
-    if (rc == LLAMA2_OK && with_sample)
-        rc = stochastic ? launch_sample_step(d, d->sampled_temperature, d->sampled_top_p, d->sampled_seed)
-                        : launch_argmax_step(d);
+    int rc = forward_fused(d, shape);
+    if (rc == LLAMA2_OK && kind == llama2_decoder::kGraphStepSampled)
+        rc = launch_sample_step(d, d->sampled_temperature, d->sampled_top_p, d->sampled_seed);
+    else if (rc == LLAMA2_OK && kind == llama2_decoder::kGraphStep)
+        rc = launch_argmax_step(d);
     ctx().capturing = false;
     hipGraph_t g = nullptr;
     hipError_t e = hipStreamEndCapture(ctx().stream, &g);
@@ -569,14 +601,39 @@ int capture(hipGraphExec_t* exec, llama2_decoder* d, bool with_sample, bool stoc
     return LLAMA2_OK;
 }
 
+// The shape for a step at `position`.  While the caller captures a graph of its own the
+// step may be replayed at any later position, so it gets the shape of the whole context.
+int step_shape(const llama2_decoder* d, int position)
+{
+    return attn_shape_index(ctx().capturing ? d->cfg.seq_len : position + 1);
+}
+
+// Launches one step of `kind`: the captured graph of that shape (captured on first use)
+// in graph mode, the same launches otherwise.
+int launch_step(llama2_decoder* d, int kind, int position)
+{
+    const int shape = step_shape(d, position);
+    if ((d->mode & LLAMA2_DECODE_GRAPH) && !ctx().capturing) {
+        hipGraphExec_t& g = d->graphs[kind][shape];
+        if (!g)
+            L2_TRY(capture(&g, d, kind, shape));
+        L2_HIP(hipGraphLaunch(g, ctx().stream));
+        return LLAMA2_OK;
+    }
+    L2_TRY(forward_fused(d, shape));
+    if (kind == llama2_decoder::kGraphStepSampled)
+        return launch_sample_step(d, d->sampled_temperature, d->sampled_top_p, d->sampled_seed);
+    if (kind == llama2_decoder::kGraphStep)
+        return launch_argmax_step(d);
+    return LLAMA2_OK;
+}
+
 void release(llama2_decoder* d)
 {
-    if (d->graph_forward)
-        (void)hipGraphExecDestroy(d->graph_forward);
-    if (d->graph_step)
-        (void)hipGraphExecDestroy(d->graph_step);
-    if (d->graph_step_sampled)
-        (void)hipGraphExecDestroy(d->graph_step_sampled);
+    for (auto& kind : d->graphs)
+        for (hipGraphExec_t g : kind)
+            if (g)
+                (void)hipGraphExecDestroy(g);
     if (d->state)
         (void)hipFree(d->state);
     if (d->attn_part)
@@ -612,7 +669,7 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
     // the block can be matched to it: 4-wavefront workgroups over 128-row blocks spread a short
     // sequence over more compute units, 16-wavefront workgroups over 512-row blocks need fewer merges.
     const bool small_blocks = seq_length <= kSmallBlockMaxSeq;
-    const int block_t = small_blocks ? 128 : kSplitT;
+    const int block_t = small_blocks ? kSmallSplitT : kSplitT;
     const int splits = ceil_div(seq_length, block_t);
     L2_CHECK(splits <= kMaxSplits, "%s: seq_length=%d exceeds %d", fn, seq_length, kMaxSplits * kSplitT);
     if (splits > 1)
@@ -622,7 +679,8 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
     a.part = ctx().attn_partials, a.counters = ctx().attn_counters, a.pos_ptr = nullptr, a.seq = seq_length;
     a.dim = dim, a.max_splits = splits, a.scale = scale;
     if (small_blocks)
-        hipLaunchKernelGGL(fused_attn_kernel<4>, dim3(splits, n_heads), dim3(256), 0, ctx().stream, a);
+        hipLaunchKernelGGL(fused_attn_kernel<kSmallWaves>, dim3(splits, n_heads), dim3(kSmallWaves * 64), 0, ctx().stream,
+                           a);
     else
         hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(splits, n_heads), dim3(kAttnWaves * 64), 0, ctx().stream, a);
     L2_LAUNCH_CHECK(fn);
@@ -703,11 +761,10 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     d->kv_dim = kv_dim;
     d->head_size = c.dim / c.n_heads;
     if (fused) {
-        d->max_splits = attn_max_splits(c.seq_len);
         hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->state), kStateBytes);
         if (e == hipSuccess)
             e = hipMalloc(reinterpret_cast<void**>(&d->attn_part),
-                          sizeof(float) * static_cast<size_t>(c.n_heads) * d->max_splits * kPartStride);
+                          sizeof(float) * static_cast<size_t>(c.n_heads) * kMaxSplits * kPartStride);
         if (e == hipSuccess)
             e = hipMalloc(reinterpret_cast<void**>(&d->counters), sizeof(unsigned) * c.n_heads);
         if (e == hipSuccess)
@@ -720,10 +777,13 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
             release(d);
             return hip_fail(e, "llama2_decode_create: scratch allocation");
         }
-        if (mode & LLAMA2_DECODE_GRAPH) {
-            int rc = capture(&d->graph_forward, d, false);
-            if (rc == LLAMA2_OK)
-                rc = capture(&d->graph_step, d, true);
+        if (mode & LLAMA2_DECODE_GRAPH) { // every shape this context can reach, so that no step pays for a capture
+            int rc = LLAMA2_OK;
+            for (int shape = 0; shape <= attn_shape_index(c.seq_len) && rc == LLAMA2_OK; ++shape) {
+                rc = capture(&d->graphs[llama2_decoder::kGraphForward][shape], d, llama2_decoder::kGraphForward, shape);
+                if (rc == LLAMA2_OK)
+                    rc = capture(&d->graphs[llama2_decoder::kGraphStep][shape], d, llama2_decoder::kGraphStep, shape);
+            }
             if (rc != LLAMA2_OK) {
                 release(d);
                 return rc;
@@ -745,11 +805,7 @@ int llama2_decode_forward(llama2_decoder* d, int position, int next_position)
     if (!(d->mode & LLAMA2_DECODE_FUSED))
         return forward_modules(d, position, next_position);
     L2_TRY(set_state(d, position, INT_MAX, 0));
-    if (d->graph_forward) {
-        L2_HIP(hipGraphLaunch(d->graph_forward, ctx().stream));
-        return LLAMA2_OK;
-    }
-    return forward_fused(d);
+    return launch_step(d, llama2_decoder::kGraphForward, position);
 }
 
 int llama2_decode_sample(llama2_decoder* d, int next_position, int generate_token, int* token)
@@ -799,27 +855,25 @@ int llama2_decode_run_sampled(llama2_decoder* d, int position, int steps, int n_
         }
         return LLAMA2_OK;
     }
-    if ((d->mode & LLAMA2_DECODE_GRAPH) && !ctx().capturing &&
-        (!d->graph_step_sampled || d->sampled_temperature != temperature || d->sampled_top_p != top_p ||
-         d->sampled_seed != seed)) {
-        // the sampling parameters are kernel arguments of the captured step: capture again when they change
-        if (d->graph_step_sampled) {
+    if (d->sampled_temperature != temperature || d->sampled_top_p != top_p || d->sampled_seed != seed) {
+        // the sampling parameters are kernel arguments of the captured steps: drop those when they change
+        bool any = false;
+        for (hipGraphExec_t g : d->graphs[llama2_decoder::kGraphStepSampled])
+            any |= g != nullptr;
+        if (any) {
+            L2_CHECK(!ctx().capturing, "%s: the sampling parameters cannot change during graph capture", fn);
             L2_HIP(hipStreamSynchronize(ctx().stream));
-            (void)hipGraphExecDestroy(d->graph_step_sampled);
-            d->graph_step_sampled = nullptr;
+            for (hipGraphExec_t& g : d->graphs[llama2_decoder::kGraphStepSampled]) {
+                if (g)
+                    (void)hipGraphExecDestroy(g);
+                g = nullptr;
+            }
         }
         d->sampled_temperature = temperature, d->sampled_top_p = top_p, d->sampled_seed = seed;
-        L2_TRY(capture(&d->graph_step_sampled, d, true, true));
     }
     L2_TRY(set_state(d, position, n_prompt, 1));
-    for (int i = 0; i < steps; ++i) {
-        if (d->graph_step_sampled && !ctx().capturing) {
-            L2_HIP(hipGraphLaunch(d->graph_step_sampled, ctx().stream));
-        } else {
-            L2_TRY(forward_fused(d));
-            L2_TRY(launch_sample_step(d, temperature, top_p, seed));
-        }
-    }
+    for (int i = 0; i < steps; ++i)
+        L2_TRY(launch_step(d, llama2_decoder::kGraphStepSampled, position + i));
     return LLAMA2_OK;
 }
 
@@ -837,14 +891,8 @@ int llama2_decode_run(llama2_decoder* d, int position, int steps, int n_prompt)
         return LLAMA2_OK;
     }
     L2_TRY(set_state(d, position, n_prompt, 1));
-    for (int i = 0; i < steps; ++i) {
-        if (d->graph_step) {
-            L2_HIP(hipGraphLaunch(d->graph_step, ctx().stream));
-        } else {
-            L2_TRY(forward_fused(d));
-            L2_TRY(launch_argmax_step(d));
-        }
-    }
+    for (int i = 0; i < steps; ++i)
+        L2_TRY(launch_step(d, llama2_decoder::kGraphStep, position + i));
     return LLAMA2_OK;
 }
 

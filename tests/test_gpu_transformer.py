@@ -106,12 +106,13 @@ def test_fused_step_tracks_module_step(oracle):
     assert_close_normwise(outs[1][1].astype(np.float64), outs[0][1].astype(np.float64), "fused vs modules K cache", 2e-3)
 
 
-@pytest.mark.parametrize("pos", [511, 512, 1100])
+@pytest.mark.parametrize("pos", [127, 128, 511, 512, 1100, 3071, 3072])
 def test_fused_step_with_long_history(oracle, pos):
-    """A step whose history spans one, two and three 512-row attention blocks:
+    """A step whose history spans 1, 2, 4, 5, 9 and 24 blocks of 128 rows and 7
+    blocks of 512 rows (the attention launch shapes either side of each change):
     the caches are filled with random rows, then one step of the module
     sequence, the fused launches, the graph replay and the oracle are compared."""
-    cfg = dict(HS128, seq_len=1200)
+    cfg = dict(HS128, seq_len=max(1200, pos + 40))
     dim, L, S = cfg["dim"], cfg["n_layers"], cfg["seq_len"]
     model = synth.random_model(cfg, seed=11, rms_random=True)
     rng = synth.rng_for(408, pos)
@@ -178,6 +179,37 @@ def test_device_resident_loop(oracle, mode):
     assert list(t.runstate.tokens.to_host(51)[1:]) == more
     ref.close()
     t.close()
+
+
+@pytest.mark.parametrize("mode", [FUSED, FUSED_GRAPH])
+def test_device_resident_loop_crosses_attention_shapes(oracle, mode):
+    """The device-resident loop picks the attention launch shape per step from the host's
+    copy of the position: run it across the changes at 128, 256 and 512 rows on top of a
+    random history and compare with single steps."""
+    cfg = dict(HS128, seq_len=600)
+    dim, L, S = cfg["dim"], cfg["n_layers"], cfg["seq_len"]
+    model = synth.random_model(cfg, seed=12)
+    for start in (122, 250, 506):
+        rng = synth.rng_for(409, start)
+        kc = synth.normal_f16(rng, L * S * dim)
+        vc = synth.normal_f16(rng, L * S * dim)
+        first = np.array([23], np.int32)
+        runs = []
+        for looped in (False, True):
+            t = Transformer(dict(cfg), model, mode=mode)
+            t.runstate.keyCache.copy_to_device(kc)
+            t.runstate.valueCache.copy_to_device(vc)
+            t.runstate.tokens.copy_to_device(first, start)
+            if looped:
+                capi.call("llama2_decode_run", t._decoder, start, 12, 0)
+            else:
+                for pos in range(start, start + 12):
+                    t.Forward(pos, pos + 1)
+                    t.Sample(pos + 1, True)
+            runs.append((t.runstate.tokens.to_host(13, start), t.runstate.logits.to_host()))
+            t.close()
+        assert np.array_equal(runs[0][0], runs[1][0]), start
+        assert np.array_equal(runs[0][1].view(np.uint16), runs[1][1].view(np.uint16)), start
 
 
 def test_generate_matches_stepwise(oracle):
