@@ -224,6 +224,11 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     VecPieces<J> gp;
     if (STAGE == STAGE_RMSNORM)
         gp.load(a.gamma, a.K);
+    // The RoPE table is requested before the weights as well: loads return in order, so a value
+    // requested after them would hold up the staging below until the first weights have arrived.
+    float rope_entry = 0.0f;
+    if (MODE == QKV_ROPE && a.rope_table && threadIdx.x < kRopeHeadSize)
+        rope_entry = a.rope_table[threadIdx.x];
     Frag<J, R> cur;
     uint16_t cur_res = 0;
     if (item < nitems)
@@ -235,7 +240,7 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     if (MODE == QKV_ROPE) {
         if (a.rope_table) { // prepared by the kernel that set the position
             if (threadIdx.x < kRopeHeadSize)
-                rope_tab[threadIdx.x] = a.rope_table[threadIdx.x];
+                rope_tab[threadIdx.x] = rope_entry;
         } else if (threadIdx.x < kRopeHeadSize / 2) {
             float c, s;
             rope_cos_sin(c, s, threadIdx.x, kRopeHeadSize, pos, a.theta);
