@@ -342,7 +342,7 @@ typedef struct llama2_decoder llama2_decoder;
 /* How llama2_decode_forward issues the step. */
 #define LLAMA2_DECODE_MODULES 0 /* the 10 module launches per layer of Transformer.Forward */
 #define LLAMA2_DECODE_FUSED 1   /* fused kernels (norm+QKV+RoPE, attention, norm+SwiGLU, ...) */
-#define LLAMA2_DECODE_GRAPH 2   /* OR-able: replay the step as a captured hipGraph          */
+#define LLAMA2_DECODE_GRAPH 2   /* OR-able: replay the step as a captured hipGraph (one per attention launch shape) */
 
 /* Binds a config, a weight set and a run state (all borrowed, all must outlive
  * the decoder) to the per-step launch sequence of Transformer.Forward
