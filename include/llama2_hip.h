@@ -377,7 +377,11 @@ int llama2_decode_run(llama2_decoder* decoder, int position, int steps, int n_pr
 /* The same loop with the stochastic sampler: the token at next_position p is
  * drawn with coin = llama2_sampler_coin(seed, p).  temperature == 0 is
  * llama2_decode_run.  (The reference draws from an unseeded System.Random,
- * src/Sampler.cs:24,42, on the host; this keeps the loop on the device.) */
+ * src/Sampler.cs:24,42, on the host; this keeps the loop on the device.)
+ * The tokens are those of llama2_decode_sample_top_p with the same coins; what
+ * state->logits and state->indices hold afterwards is not: when a short head of
+ * the sorted distribution carries more than top_p of the mass, only that head
+ * is sorted and summed. */
 int llama2_decode_run_sampled(llama2_decoder* decoder, int position, int steps, int n_prompt,
                               float temperature, float top_p, unsigned long long seed);
 int llama2_decode_destroy(llama2_decoder* decoder);

@@ -363,7 +363,7 @@ __device__ __forceinline__ void sample_step(const SampleStepArgs& a, SamplerLds&
         write_rope_table(a.state, threadIdx.x - 64, pos0 + 1, a.theta); // for the next step
     if (pos0 + 1 >= n_prompt) { // uniform over the workgroup
         const float coin = sampler_coin(a.seed, pos0 + 1);
-        const int token = sample_dev<LDS_SORT ? 4 : 8, LDS_SORT>(a.logits, a.indices, a.size, a.temperature, a.top_p,
+        const int token = sample_dev<LDS_SORT ? 4 : 8, LDS_SORT, true>(a.logits, a.indices, a.size, a.temperature, a.top_p,
                                                                  coin, a.keys2, a.values2, lds, buf);
         if (threadIdx.x == 0)
             a.tokens[pos0 + 1] = token;

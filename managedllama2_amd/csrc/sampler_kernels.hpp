@@ -338,27 +338,13 @@ __device__ __forceinline__ uint16_t sort_key_of_rank(uint32_t rank)
     return static_cast<uint16_t>((rank & 0x8000u) ? rank ^ 0x8000u : ~rank);
 }
 
-// IDENTITY: values[i] == i on entry (as softmax_logits leaves them), so the
-// sorted payload is the original position itself and no gather is needed.
-template <bool IDENTITY>
-__device__ __forceinline__ void sort_lds_dev(uint16_t* keys, int* values, int size, SamplerLds& lds, SortLds& buf)
+// The four passes over items held C per thread (thread t owns positions C*t .. C*t + C - 1;
+// C = 32 is the full vocabulary, smaller C a short list).  On return the thread holds the
+// sorted items of its positions.
+template <int C>
+__device__ __forceinline__ void sort_passes(uint32_t (&it)[C], bool active, SamplerLds& lds, SortLds& buf)
 {
-    const int first = threadIdx.x * 32;
-    const bool active = first < size; // threads beyond the (padded) input own nothing
-    uint32_t it[32];
-    if (active) {
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            uint16_t kb[8];
-            load_bits8(kb, keys, first + c * 8, size);
-#pragma unroll
-            for (int k = 0; k < 8; ++k) {
-                const int idx = first + c * 8 + k;
-                // padding up to the thread's 32 items: smallest rank, behind every real item (stable)
-                it[c * 8 + k] = (idx < size ? sort_rank(kb[k]) << 16 : 0u) | static_cast<uint32_t>(idx);
-            }
-        }
-    }
+    const int first = threadIdx.x * C;
     // Between the read-back of one pass and the scatter of the next the item
     // buffer is idle: its first 16 x 1024 words serve as 32-bit (bucket, thread)
     // counters, filled with fire-and-forget LDS adds.
@@ -372,7 +358,7 @@ __device__ __forceinline__ void sort_lds_dev(uint16_t* keys, int* values, int si
         // own words only: no barrier needed before the adds below
         if (active) {
 #pragma unroll
-            for (int k = 0; k < 32; ++k) {
+            for (int k = 0; k < C; ++k) {
                 const uint32_t d = 15u - ((it[k] >> shift) & 15u); // bucket 0 = largest digit
                 __hip_atomic_fetch_add(&cnt32[d * kSampBlock + threadIdx.x], 1u, __ATOMIC_RELAXED,
                                        __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -412,7 +398,7 @@ __device__ __forceinline__ void sort_lds_dev(uint16_t* keys, int* values, int si
             const uint32_t one = (threadIdx.x & 1) ? 0x10000u : 1u;
             const int hshift = (threadIdx.x & 1) * 16;
 #pragma unroll
-            for (int k = 0; k < 32; ++k) {
+            for (int k = 0; k < C; ++k) {
                 const uint32_t d = 15u - ((it[k] >> shift) & 15u);
                 const uint32_t old = __hip_atomic_fetch_add(&words[(d * kSampBlock + threadIdx.x) >> 1], one,
                                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -425,11 +411,41 @@ __device__ __forceinline__ void sort_lds_dev(uint16_t* keys, int* values, int si
         __syncthreads();
         if (active) {
 #pragma unroll
-            for (int k = 0; k < 32; ++k)
+            for (int k = 0; k < C; ++k)
                 it[k] = buf.item[sort_slot(first + k)];
         }
         __syncthreads(); // everyone has its items back before the buffer turns into counters again
     }
+}
+
+// The thread's 32 consecutive keys as sort items: (rank << 16) | position.
+__device__ __forceinline__ void sort_load_items(uint32_t (&it)[32], const uint16_t* keys, int size)
+{
+    const int first = threadIdx.x * 32;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        uint16_t kb[8];
+        load_bits8(kb, keys, first + c * 8, size);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int idx = first + c * 8 + k;
+            // padding up to the thread's 32 items: smallest rank, behind every real item (stable)
+            it[c * 8 + k] = (idx < size ? sort_rank(kb[k]) << 16 : 0u) | static_cast<uint32_t>(idx);
+        }
+    }
+}
+
+// IDENTITY: values[i] == i on entry (as softmax_logits leaves them), so the
+// sorted payload is the original position itself and no gather is needed.
+template <bool IDENTITY>
+__device__ __forceinline__ void sort_lds_dev(uint16_t* keys, int* values, int size, SamplerLds& lds, SortLds& buf)
+{
+    const int first = threadIdx.x * 32;
+    const bool active = first < size; // threads beyond the (padded) input own nothing
+    uint32_t it[32];
+    if (active)
+        sort_load_items(it, keys, size);
+    sort_passes<32>(it, active, lds, buf);
     if (active) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
@@ -478,6 +494,160 @@ __device__ __forceinline__ void sort_lds_dev(uint16_t* keys, int* values, int si
         }
     }
     __syncthreads(); // the sorted arrays are visible to the whole workgroup
+}
+
+// ---- the head of the sorted order only ------------------------------------------------
+// Sampler.Sample (src/Sampler.cs:56-66) reads the sorted probabilities only up to the first
+// position whose cumulative sum reaches coin * topP < topP.  When the largest probabilities
+// alone add up to more than topP, sorting them is enough: the head of a stable sort does not
+// depend on the tail, and neither do the prefix sums over it.
+//
+// The keys must be probabilities (fp16 in [0, 1]).  Each is put in a bucket by how many
+// binades it lies below the largest one (subnormals included: most of a 32000-entry
+// distribution is subnormal in fp16); the exact mass of every bucket (integers in units
+// of 2^-24, the smallest fp16 subnormal) tells how many buckets are needed to reach `need`;
+// their items are compacted in input order, sorted C <= 16 per thread and written to the head
+// of keys / values (values[i] == i on entry).  Returns the length n of that head, whose exact
+// sum is at least `need`, or 0 when it did nothing (no such head within 15 binades and half
+// the buffer, or keys that are no probabilities): then the caller sorts everything.
+template <int C>
+__device__ __noinline__ void sort_head_finish(uint16_t* keys, int* values, int n, SamplerLds* lds, SortLds* buf)
+{
+    const int first = threadIdx.x * C;
+    const bool active = first < n;
+    uint32_t it[C];
+#pragma unroll
+    for (int k = 0; k < C; ++k) {
+        const int p = first + k;
+        it[k] = (active && p < n) ? buf->item[sort_slot(p)] : static_cast<uint32_t>(p & 0xFFFF);
+    }
+    __syncthreads(); // the compacted items are in registers before the buffer turns into counters
+    sort_passes<C>(it, active, *lds, *buf);
+#pragma unroll
+    for (int k = 0; k < C; ++k) {
+        const int p = first + k;
+        if (active && p < n) {
+            keys[p] = sort_key_of_rank(it[k] >> 16);
+            values[p] = static_cast<int>(it[k] & 0xFFFFu);
+        }
+    }
+    __syncthreads();
+}
+
+// Binade of a non-negative fp16 key: the exponent field for normal numbers, continued downwards
+// through the subnormals by the position of the leading mantissa bit (zero: below all of them).
+__device__ __forceinline__ int sort_head_binade(uint32_t rank)
+{
+    const int e = static_cast<int>((rank >> 10) & 31u);
+    const uint32_t mant = rank & 0x3FFu;
+    return e ? e : (mant ? 22 - __clz(mant) : -10); // mant in [2^k, 2^(k+1)): k - 9
+}
+
+__device__ __forceinline__ int sort_head_bucket(uint32_t item, int emax)
+{
+    const uint32_t r = item >> 16;
+    const int below = emax - sort_head_binade(r);
+    return (r < 0x8000u || below > 15) ? 15 : below; // padding and negative keys: last bucket
+}
+
+__device__ __noinline__ int sort_head_call(uint16_t* keys, int* values, int size, float need, SamplerLds* lds_,
+                                           SortLds* buf_)
+{
+    SamplerLds& lds = *lds_;
+    SortLds& buf = *buf_;
+    const bool active = static_cast<int>(threadIdx.x) * 32 < size;
+    uint32_t it[32];
+    int top = 0;
+    if (active) {
+        sort_load_items(it, keys, size);
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            top = max(top, static_cast<int>(it[k] >> 16));
+    }
+    top = 0xFFFF - samp_block_min(0xFFFF - top, lds.redi);
+    if (top > 0xBC00 || top < 0x8000) // something above 1.0 (or NaN), or nothing positive
+        return 0;
+    const int emax = sort_head_binade(static_cast<uint32_t>(top));
+    uint32_t* mass = buf.item; // [16][kSampBlock], own words only
+#pragma unroll
+    for (int d = 0; d < 16; ++d)
+        mass[d * kSampBlock + threadIdx.x] = 0u;
+    if (active) {
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            const uint32_t r = it[k] >> 16;
+            const uint32_t e = (r >> 10) & 31u, mant = r & 0x3FFu;
+            uint32_t units = e ? (0x400u | mant) << (e - 1) : mant; // value * 2^24, exact
+            if (r < 0x8000u)
+                units = 0u;
+            __hip_atomic_fetch_add(&mass[sort_head_bucket(it[k], emax) * kSampBlock + threadIdx.x], units,
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        }
+    }
+    __syncthreads();
+    {
+        // wavefront d adds up bucket d: 64 lanes x 16 consecutive words
+        const u32x4* mine = reinterpret_cast<const u32x4*>(mass + threadIdx.x * 16);
+        uint32_t sum = 0;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const u32x4 m4 = mine[q];
+            sum += m4[0] + m4[1] + m4[2] + m4[3];
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1)
+            sum += __shfl_xor(sum, off, 64);
+        if ((threadIdx.x & 63) == 0)
+            lds.redi[threadIdx.x >> 6] = static_cast<int>(sum); // the whole vocabulary stays below 2^31 units
+    }
+    __syncthreads();
+    const float need_units = ceilf(need * 16777216.0f);
+    int last_bucket = -1;
+    {
+        float cum = 0.0f; // sums of integers below 2^25 in fp32 lose at most a unit or two: `need` carries a margin
+#pragma unroll
+        for (int d = 0; d < 15; ++d) {
+            cum += static_cast<float>(lds.redi[d]);
+            if (last_bucket < 0 && cum >= need_units)
+                last_bucket = d;
+        }
+    }
+    __syncthreads();
+    if (last_bucket < 0)
+        return 0;
+    int keep = 0;
+    if (active) {
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            keep += sort_head_bucket(it[k], emax) <= last_bucket;
+    }
+    const int before = samp_block_exclusive_scan<int>(keep, lds.redi);
+    if (threadIdx.x == kSampBlock - 1)
+        lds.redi[0] = before + keep;
+    __syncthreads();
+    const int n = lds.redi[0];
+    __syncthreads();
+    if (n > kSortLdsThreads * 16)
+        return 0;
+    if (active) {
+        int at = before;
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            if (sort_head_bucket(it[k], emax) <= last_bucket)
+                buf.item[sort_slot(at++)] = it[k];
+    }
+    __syncthreads();
+    if (n <= kSortLdsThreads)
+        sort_head_finish<1>(keys, values, n, lds_, buf_);
+    else if (n <= kSortLdsThreads * 2)
+        sort_head_finish<2>(keys, values, n, lds_, buf_);
+    else if (n <= kSortLdsThreads * 4)
+        sort_head_finish<4>(keys, values, n, lds_, buf_);
+    else if (n <= kSortLdsThreads * 8)
+        sort_head_finish<8>(keys, values, n, lds_, buf_);
+    else
+        sort_head_finish<16>(keys, values, n, lds_, buf_);
+    return n;
 }
 
 // ---- cumulative_sum (native/cumulative_sum_kernel.cu:8-26) ---------------------------
@@ -579,23 +749,34 @@ __device__ __noinline__ void cumulative_sum_call(uint16_t* values, int size, Sam
     cumulative_sum_dev<CH>(values, size, *lds);
 }
 
-template <int CH, bool LDS_SORT>
+// HEAD_ONLY: the caller needs the token alone, not the sorted arrays and their prefix sums: when a
+// short head of the sorted order holds more than top_p of the mass, only that head is sorted and
+// summed (the token is the same; what logits / indices hold afterwards is not).
+template <int CH, bool LDS_SORT, bool HEAD_ONLY = false>
 __device__ __forceinline__ int sample_dev(uint16_t* logits, int* indices, int size, float temperature, float top_p,
                                           float coin, uint16_t* keys2, int* values2, SamplerLds& lds, SortLds* buf)
 {
     softmax_logits_call<CH>(logits, size, temperature, indices, &lds);
     __syncthreads();
     float threshold = coin;
+    int n = size;
     if (!(top_p <= 0.0f || top_p >= 1.0f)) {
-        if (LDS_SORT)
+        // The prefix sums are rounded to fp16 (2^-11) after a blocked fp32 summation (a few 2^-24):
+        // a head whose exact mass is 1.004 top_p reaches top_p > coin * top_p in that arithmetic too.
+        int head = 0;
+        if (LDS_SORT && HEAD_ONLY)
+            head = sort_head_call(logits, indices, size, top_p * 1.004f, &lds, buf);
+        if (head)
+            n = head;
+        else if (LDS_SORT)
             sort_lds_identity_call(logits, indices, size, &lds, buf); // indices are 0..size-1 here
         else
             sort_call<CH>(logits, indices, size, keys2, values2, &lds);
         threshold = coin * top_p;
     }
-    cumulative_sum_call<CH>(logits, size, &lds);
+    cumulative_sum_call<CH>(logits, n, &lds);
     __syncthreads();
-    return sample_top_p_dev<CH>(logits, indices, size, threshold, lds);
+    return sample_top_p_dev<CH>(logits, indices, n, threshold, lds);
 }
 
 } // namespace l2
