@@ -360,9 +360,11 @@ int llama2_decode_forward(llama2_decoder* decoder, int position, int next_positi
 int llama2_decode_sample(llama2_decoder* decoder, int next_position, int generate_token,
                          int* token);
 /* Sampler.Sample with temperature and top-p (src/Sampler.cs:40-70): the greedy
- * branch when temperature == 0 or !generate_token, otherwise llama2_sample on
- * state->logits / state->indices with the caller's uniform `coin` in [0, 1);
- * then reads tokens[next_position] back. */
+ * branch when temperature == 0 or !generate_token, otherwise the token that
+ * llama2_sample picks on state->logits / state->indices with the caller's
+ * uniform `coin` in [0, 1); then reads tokens[next_position] back.  Only the
+ * token is defined: the sort stops at the head of the distribution that holds
+ * top_p of the mass, so logits / indices are left partly sorted. */
 int llama2_decode_sample_top_p(llama2_decoder* decoder, int next_position, int generate_token,
                                float temperature, float top_p, float coin, int* token);
 /* The uniform number the device-resident sampling loop draws for the token at

@@ -35,6 +35,10 @@ Context& ctx();
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char* what);
 int ensure_attn_partials(size_t bytes);
+// Sampler.Sample's stochastic branch in one launch (sampler.hip).  token_only: the caller reads the
+// token alone, so the sort may stop at the head of the distribution that holds top_p of the mass.
+int sample_launch(const char* fn, uint16_t* logits, int* indices, int size, float temperature, float top_p, float coin,
+                  int* result, int pos, bool token_only);
 
 #define L2_REQUIRE_INIT()                                                          \
     do {                                                                           \

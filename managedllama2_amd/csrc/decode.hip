@@ -828,8 +828,8 @@ int llama2_decode_sample_top_p(llama2_decoder* d, int next_position, int generat
         return llama2_decode_sample(d, next_position, generate_token, token);
     L2_CHECK(next_position >= 0 && next_position <= d->cfg.seq_len, "%s: next_position=%d", fn, next_position);
     L2_TRY(check_sampling(fn, d, temperature));
-    L2_TRY(llama2_sample(d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p, coin, d->s.tokens,
-                         next_position)); // :50-66
+    L2_TRY(sample_launch(fn, d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p, coin, d->s.tokens,
+                         next_position, true)); // :50-66
     return llama2_memcpy_d2h(token, d->s.tokens, static_cast<size_t>(next_position) * sizeof(int), sizeof(int)); // :69
 }
 
@@ -850,8 +850,8 @@ int llama2_decode_run_sampled(llama2_decoder* d, int position, int steps, int n_
         for (int pos = position; pos < position + steps; ++pos) {
             L2_TRY(forward_modules(d, pos, pos + 1));
             if (pos + 1 >= n_prompt)
-                L2_TRY(llama2_sample(d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p,
-                                     sampler_coin(seed, pos + 1), d->s.tokens, pos + 1));
+                L2_TRY(sample_launch(fn, d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p,
+                                     sampler_coin(seed, pos + 1), d->s.tokens, pos + 1, true));
         }
         return LLAMA2_OK;
     }

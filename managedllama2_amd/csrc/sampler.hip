@@ -47,12 +47,14 @@ __global__ __launch_bounds__(kSampBlock) void sample_top_p_kernel(const uint16_t
         result[pos] = token;
 }
 
+template <bool HEAD_ONLY>
 __global__ __launch_bounds__(kSampBlock) void sample_kernel(uint16_t* logits, int* indices, int size, float temperature,
                                                             float top_p, float coin, int* result, int pos)
 {
     __shared__ SamplerLds lds;
     __shared__ SortLds buf;
-    const int token = sample_dev<4, true>(logits, indices, size, temperature, top_p, coin, nullptr, nullptr, lds, &buf);
+    const int token =
+        sample_dev<4, true, HEAD_ONLY>(logits, indices, size, temperature, top_p, coin, nullptr, nullptr, lds, &buf);
     if (threadIdx.x == 0)
         result[pos] = token;
 }
@@ -155,16 +157,28 @@ int llama2_sample(llama2_half* logits, int* indices, int size, float temperature
                   int* result, int pos)
 {
     L2_REQUIRE_INIT();
-    const char* fn = "llama2_sample";
+    return sample_launch("llama2_sample", logits, indices, size, temperature, top_p, coin, result, pos, false);
+}
+
+} // extern "C"
+
+namespace l2 {
+
+int sample_launch(const char* fn, uint16_t* logits, int* indices, int size, float temperature, float top_p, float coin,
+                  int* result, int pos, bool token_only)
+{
     L2_CHECK(logits && indices && result, "%s: null pointer", fn);
     L2_TRY(check_sampler_size(fn, size));
     L2_CHECK(temperature > 0.0f, "%s: temperature=%g must be positive (temperature 0 is the argmax branch)", fn,
              static_cast<double>(temperature));
     L2_CHECK(pos >= 0, "%s: pos=%d is negative", fn, pos);
     L2_CHECK(aligned(logits, 16) && aligned(indices, 16), "%s: logits and indices must be 16-byte aligned", fn);
-    if (size <= kSortLdsItems)
-        hipLaunchKernelGGL(sample_kernel, dim3(1), dim3(kSampBlock), 0, ctx().stream, logits, indices, size, temperature,
-                           top_p, coin, result, pos);
+    if (size <= kSortLdsItems && token_only)
+        hipLaunchKernelGGL(sample_kernel<true>, dim3(1), dim3(kSampBlock), 0, ctx().stream, logits, indices, size,
+                           temperature, top_p, coin, result, pos);
+    else if (size <= kSortLdsItems)
+        hipLaunchKernelGGL(sample_kernel<false>, dim3(1), dim3(kSampBlock), 0, ctx().stream, logits, indices, size,
+                           temperature, top_p, coin, result, pos);
     else
         hipLaunchKernelGGL(sample_big_kernel, dim3(1), dim3(kSampBlock), 0, ctx().stream, logits, indices, size,
                            temperature, top_p, coin, result, pos, ctx().sort_keys, ctx().sort_values);
@@ -172,4 +186,4 @@ int llama2_sample(llama2_half* logits, int* indices, int size, float temperature
     return LLAMA2_OK;
 }
 
-} // extern "C"
+} // namespace l2

@@ -33,7 +33,9 @@ class CoinStream:
         return lib_coin(self.seed, self.pos)
 
 
-def stepwise(model, mode, prompt, steps, temperature=T, top_p=TOP_P, seed=SEED, cfg=CFG):
+def stepwise(model, mode, prompt, steps, temperature=T, top_p=TOP_P, seed=SEED, cfg=CFG, module_sampler=False):
+    """Forward + Sample per token with a read-back, as Transformer.Generate does.  module_sampler: sample with
+    the four sampler modules (which sort the whole vocabulary) even when a decoder runs the forward step."""
     coins = CoinStream(seed)
     t = Transformer(dict(cfg), model, mode=mode, temperature=temperature, topP=top_p, random=coins)
     t.runstate.tokens.copy_to_device(np.array(prompt, np.int32))
@@ -42,7 +44,7 @@ def stepwise(model, mode, prompt, steps, temperature=T, top_p=TOP_P, seed=SEED, 
         t.Forward(pos, pos + 1)
         coins.pos = pos + 1
         gen = pos + 1 >= len(prompt)
-        tok = t.Sample(pos + 1, gen)
+        tok = t.sampler.Sample(pos + 1, gen) if module_sampler else t.Sample(pos + 1, gen)
         out.append(tok)
     t.close()
     return out
@@ -98,15 +100,18 @@ def test_device_resident_sampling_loop(mode):
 
 @pytest.mark.parametrize("temperature", [0.05, 0.3, 1.0, 3.0, 30.0])
 def test_device_loop_sorts_only_what_it_needs(temperature):
-    """The device-resident loop sorts only the head of the distribution that holds more than top_p of
-    the mass (and everything when there is no short head); the host loop sorts all 32000 entries.
-    From peaked (a handful of candidates) to flat (no short head) the tokens must be the same."""
+    """The decoder's samplers (one launch per token, and the device-resident loop) sort only the head of
+    the distribution that holds more than top_p of the mass, and everything when there is no short head;
+    the sampler modules sort all 32000 entries.  From peaked (a handful of candidates) to flat (no short
+    head) the tokens must be the same."""
     cfg = dict(CFG, vocab_size=32000, n_layers=1)
     model = synth.random_model(cfg, seed=38, rms_random=True)
     prompt = [int(t) for t in synth.rng_for(605).integers(3, cfg["vocab_size"], 3)]
     t = Transformer(dict(cfg), model, mode=FUSED_GRAPH)
     for top_p in (0.02, 0.5, 0.9, 0.99, 0.9999):
-        want = stepwise(model, FUSED_GRAPH, prompt, 20, temperature=temperature, top_p=top_p, seed=11, cfg=cfg)
+        want = stepwise(model, FUSED_GRAPH, prompt, 20, temperature=temperature, top_p=top_p, seed=11, cfg=cfg,
+                        module_sampler=True)
+        assert want == stepwise(model, FUSED_GRAPH, prompt, 20, temperature=temperature, top_p=top_p, seed=11, cfg=cfg)
         t.runstate.tokens.copy_to_device(np.array(prompt + [0] * 40, np.int32))
         capi.call("llama2_decode_run_sampled", t._decoder, 0, 20, len(prompt), temperature, top_p, 11)
         assert list(t.runstate.tokens.to_host(21)[1:]) == want, (temperature, top_p)
