@@ -232,16 +232,33 @@ __global__ __launch_bounds__(kThreads) void vecmat_kernel(uint16_t* out, float* 
     }
 }
 
-__global__ void vecmat_reduce_kernel(uint16_t* out, const float* partials, int rows, int o_stride, int n_heads,
-                                     int splits)
+// One workgroup adds up 64 consecutive outputs: wavefront w takes the splits w, w + 16, ... (one
+// coalesced 256-byte row of partials each, independent loads), then the 16 wavefront sums are
+// added in wavefront order (fixed association: deterministic).
+constexpr int kReduceWaves = 16;
+__global__ __launch_bounds__(kReduceWaves * 64) void vecmat_reduce_kernel(uint16_t* out, const float* partials,
+                                                                          int rows, int o_stride, int n_heads,
+                                                                          int splits)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n_heads * rows)
-        return;
+    __shared__ float red[kReduceWaves][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int total = n_heads * rows;
+    const int i = blockIdx.x * 64 + lane;
     float s = 0.0f;
-    for (int k = 0; k < splits; ++k)
-        s += partials[static_cast<size_t>(k) * n_heads * rows + i];
-    out[static_cast<size_t>(i / rows) * o_stride + (i % rows)] = float_to_half_bits(s);
+    if (i < total) {
+#pragma unroll 8
+        for (int k = wave; k < splits; k += kReduceWaves)
+            s += partials[static_cast<size_t>(k) * total + i];
+    }
+    red[wave][lane] = s;
+    __syncthreads();
+    if (wave == 0 && i < total) {
+        float t = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kReduceWaves; ++w)
+            t += red[w][lane];
+        out[static_cast<size_t>(i / rows) * o_stride + (i % rows)] = float_to_half_bits(t);
+    }
 }
 
 // Any shape / stride: one thread per output element.
@@ -352,7 +369,7 @@ int llama2_vec_mat(llama2_half* output, const llama2_half* vector, const llama2_
                            matrix, rows, cols, m_col_stride, o_stride, m_row_stride, n_heads, t_per_wg);
         L2_LAUNCH_CHECK(fn);
         if (splits > 1) {
-            hipLaunchKernelGGL(vecmat_reduce_kernel, dim3(ceil_div(n_heads * rows, 256)), dim3(256), 0,
+            hipLaunchKernelGGL(vecmat_reduce_kernel, dim3(ceil_div(n_heads * rows, 64)), dim3(kReduceWaves * 64), 0,
                                ctx().stream, output, partials, rows, o_stride, n_heads, splits);
             L2_LAUNCH_CHECK("vecmat_reduce_kernel");
         }
