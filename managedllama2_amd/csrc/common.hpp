@@ -233,6 +233,70 @@ struct VecPieces {
     }
 };
 
+// Largest fp16 value of x[0..size), lowest index among equals, by a workgroup of 1024 threads;
+// valid in thread 0 (0 when every entry is NaN).  A candidate is the pair (value, index); `better`
+// is a strict total order, so every reduction order yields the same winner (no race, unlike
+// native/argmax_kernel.cu:32-36).  `sv`, `si`: 16 entries of LDS each.
+__device__ __forceinline__ bool better(float va, int ia, float vb, int ib)
+{
+    return va > vb || (va == vb && ia < ib);
+}
+
+__device__ __forceinline__ int block1024_argmax(const uint16_t* x, int size, float* sv, int* si)
+{
+    float bv = -INFINITY;
+    int bi = 0x7FFFFFFF;
+    // 16 bytes per load while whole groups of 8 remain (when x is 16-byte aligned), the rest one by one
+    const int n8 = (reinterpret_cast<uintptr_t>(x) & 15) == 0 ? size >> 3 : 0;
+    for (int g = threadIdx.x; g < n8; g += 1024) {
+        const u32x4 v = reinterpret_cast<const u32x4*>(x)[g];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float f = half_bits_to_float(static_cast<uint16_t>(v[k >> 1] >> (16 * (k & 1))));
+            if (better(f, g * 8 + k, bv, bi)) {
+                bv = f;
+                bi = g * 8 + k;
+            }
+        }
+    }
+    for (int i = n8 * 8 + threadIdx.x; i < size; i += 1024) {
+        const float f = half_bits_to_float(x[i]);
+        if (better(f, i, bv, bi)) {
+            bv = f;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const float ov = __shfl_xor(bv, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (better(ov, oi, bv, bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if ((threadIdx.x & 63) == 0) {
+        sv[threadIdx.x >> 6] = bv;
+        si[threadIdx.x >> 6] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x < 64) {
+        bv = threadIdx.x < 16 ? sv[threadIdx.x] : -INFINITY;
+        bi = threadIdx.x < 16 ? si[threadIdx.x] : 0x7FFFFFFF;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oi = __shfl_xor(bi, off, 64);
+            if (better(ov, oi, bv, bi)) {
+                bv = ov;
+                bi = oi;
+            }
+        }
+    }
+    return bi == 0x7FFFFFFF ? 0 : bi;
+}
+
 #endif // __HIPCC__
+
 
 } // namespace l2

@@ -266,11 +266,6 @@ __global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance,
         write_rope_table(state, threadIdx.x, pos, theta);
 }
 
-__device__ __forceinline__ bool better(float va, int ia, float vb, int ib)
-{
-    return va > vb || (va == vb && ia < ib);
-}
-
 // Sampler.Sample greedy branch (src/Sampler.cs:44-47) against the device state:
 // tokens[pos+1] = argmax(logits) iff pos+1 >= n_prompt; lowest index wins ties.
 __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, int size, int* tokens, int* state,
@@ -281,61 +276,12 @@ __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, in
     const int pos0 = state[0], advance0 = state[2]; // read by every thread before thread 0 updates them
     if (advance0 && threadIdx.x >= 64 && threadIdx.x < 64 + kRopeHeadSize / 2)
         write_rope_table(state, threadIdx.x - 64, pos0 + 1, theta); // for the next step
-    float bv = -INFINITY;
-    int bi = INT_MAX;
-    // 16 bytes per load while whole groups of 8 remain (x is 16-byte aligned:
-    // checked on the host), the last size % 8 elements one by one
-    const int n8 = size >> 3;
-    for (int g = threadIdx.x; g < n8; g += 1024) {
-        const u32x4 v = reinterpret_cast<const u32x4*>(x)[g];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const float f = half_bits_to_float(static_cast<uint16_t>(v[k >> 1] >> (16 * (k & 1))));
-            if (better(f, g * 8 + k, bv, bi)) {
-                bv = f;
-                bi = g * 8 + k;
-            }
-        }
-    }
-    for (int i = n8 * 8 + threadIdx.x; i < size; i += 1024) {
-        const float f = half_bits_to_float(x[i]);
-        if (better(f, i, bv, bi)) {
-            bv = f;
-            bi = i;
-        }
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, 64);
-        const int oi = __shfl_xor(bi, off, 64);
-        if (better(ov, oi, bv, bi)) {
-            bv = ov;
-            bi = oi;
-        }
-    }
-    if ((threadIdx.x & 63) == 0) {
-        sv[threadIdx.x >> 6] = bv;
-        si[threadIdx.x >> 6] = bi;
-    }
-    __syncthreads();
-    if (threadIdx.x < 64) {
-        bv = threadIdx.x < 16 ? sv[threadIdx.x] : -INFINITY;
-        bi = threadIdx.x < 16 ? si[threadIdx.x] : INT_MAX;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(bv, off, 64);
-            const int oi = __shfl_xor(bi, off, 64);
-            if (better(ov, oi, bv, bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
-        if (threadIdx.x == 0) {
-            if (pos0 + 1 >= state[1])
-                tokens[pos0 + 1] = bi == INT_MAX ? 0 : bi;
-            if (advance0)
-                state[0] = pos0 + 1;
-        }
+    const int best = block1024_argmax(x, size, sv, si);
+    if (threadIdx.x == 0) {
+        if (pos0 + 1 >= state[1])
+            tokens[pos0 + 1] = best;
+        if (advance0)
+            state[0] = pos0 + 1;
     }
 }
 

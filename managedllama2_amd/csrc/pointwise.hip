@@ -124,57 +124,16 @@ __global__ __launch_bounds__(kBlock) void softmax_kernel(uint16_t* v, int size)
         row[i] = float_to_half_bits(buf[i] / sum);
 }
 
-// Largest logit, lowest index among equals.  A candidate is the pair
-// (value, index); `better` is a strict total order so every reduction order
-// yields the same winner (no race, unlike native/argmax_kernel.cu:32-36).
-__device__ __forceinline__ bool better(float va, int ia, float vb, int ib)
-{
-    return va > vb || (va == vb && ia < ib);
-}
-
+// Largest logit, lowest index among equals (test/ArgmaxTests.cs:33-46).
+static_assert(kBlock == 1024, "block1024_argmax");
 __global__ __launch_bounds__(kBlock) void argmax_kernel(const uint16_t* x, int size, int* result, int pos,
                                                         int write_token)
 {
     __shared__ float sv[kBlockWaves];
     __shared__ int si[kBlockWaves];
-    float bv = -INFINITY;
-    int bi = 0x7FFFFFFF;
-    for (int i = threadIdx.x; i < size; i += kBlock) {
-        const float f = half_bits_to_float(x[i]);
-        if (better(f, i, bv, bi)) {
-            bv = f;
-            bi = i;
-        }
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, 64);
-        const int oi = __shfl_xor(bi, off, 64);
-        if (better(ov, oi, bv, bi)) {
-            bv = ov;
-            bi = oi;
-        }
-    }
-    if ((threadIdx.x & 63) == 0) {
-        sv[threadIdx.x >> 6] = bv;
-        si[threadIdx.x >> 6] = bi;
-    }
-    __syncthreads();
-    if (threadIdx.x < 64) {
-        bv = threadIdx.x < kBlockWaves ? sv[threadIdx.x] : -INFINITY;
-        bi = threadIdx.x < kBlockWaves ? si[threadIdx.x] : 0x7FFFFFFF;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(bv, off, 64);
-            const int oi = __shfl_xor(bi, off, 64);
-            if (better(ov, oi, bv, bi)) {
-                bv = ov;
-                bi = oi;
-            }
-        }
-        if (threadIdx.x == 0 && write_token)
-            result[pos] = bi == 0x7FFFFFFF ? 0 : bi; // all-NaN input: index 0
-    }
+    const int best = block1024_argmax(x, size, sv, si);
+    if (threadIdx.x == 0 && write_token)
+        result[pos] = best;
 }
 
 __global__ void embedding_kernel(uint16_t* out, const uint16_t* table, int size, const int* tokens, int pos)

@@ -158,6 +158,24 @@ class TestArgmax:
         x[31999] = -2.0
         assert self.Argmax(x, 32000) == 31999
 
+    def test_ragged_sizes_and_unaligned_input(self, oracle):
+        # 16-byte loads over whole groups of 8, the remainder one by one; an input that is not
+        # 16-byte aligned takes the element-wise path altogether
+        rng = synth.rng_for(334)
+        for n in (1, 7, 8, 9, 1023, 1024, 8191, 8195, 32003):
+            x = synth.normal_f16(rng, n + 3, 1.0)
+            d = up(x)
+            result = up(np.full(1, -7, np.int32))
+            for off in (0, 1, 3):
+                want = oracle.ref_argmax(x[off:off + n])
+                capi.call("llama2_argmax", d.ptr + 2 * off, n, result.ptr, 0, 1)
+                assert int(result[0]) == want == int(np.argmax(x[off:off + n])), (n, off)
+                x2 = x.copy()
+                x2[off + n - 1] = 100.0  # the winner in the tail
+                d2 = up(x2)
+                capi.call("llama2_argmax", d2.ptr + 2 * off, n, result.ptr, 0, 1)
+                assert int(result[0]) == n - 1, (n, off)
+
     def test_write_token_flag_and_position(self):
         rng = synth.rng_for(333)
         x = f16(rng.random(100))
