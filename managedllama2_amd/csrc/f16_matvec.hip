@@ -232,6 +232,66 @@ __global__ __launch_bounds__(kThreads) void vecmat_kernel(uint16_t* out, float* 
     }
 }
 
+// Short sequences of 128-wide heads (cols <= 512): one workgroup of 16 wavefronts per head and no
+// partial sums in memory.  16 lanes share a timestep (16 bytes of its value row each), the 64 groups
+// take the timesteps round-robin, every load is issued before the first use, and the groups are
+// combined in a fixed order (within the wavefront by shuffles, across wavefronts through LDS).
+constexpr int kHeadVecMatCols = 512;
+__global__ __launch_bounds__(1024) void vecmat_head_kernel(uint16_t* out, const uint16_t* att, const uint16_t* V,
+                                                           int cols, int m_col_stride, int o_stride,
+                                                           int m_row_stride)
+{
+    constexpr int PASSES = kHeadVecMatCols / 64;
+    __shared__ float red[16][128];
+    const int h = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int l16 = lane & 15, grp = wave * 4 + (lane >> 4);
+    const uint16_t* vbase = V + static_cast<size_t>(h) * m_col_stride + l16 * 8;
+    const uint16_t* abase = att + static_cast<size_t>(h) * cols;
+    u32x4 vv[PASSES];
+    float a[PASSES];
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+        const int t = i * 64 + grp;
+        const bool ok = t < cols;
+        vv[i] = ok ? __builtin_nontemporal_load(
+                         reinterpret_cast<const u32x4*>(vbase + static_cast<size_t>(t) * m_row_stride))
+                   : u32x4{0u, 0u, 0u, 0u};
+        a[i] = ok ? half_bits_to_float(abase[t]) : 0.0f;
+    }
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+        acc[k] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const h2_t p = as_h2(vv[i][k]);
+            acc[2 * k] += a[i] * static_cast<float>(p[0]);
+            acc[2 * k + 1] += a[i] * static_cast<float>(p[1]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        acc[k] += __shfl_xor(acc[k], 16, 64);
+        acc[k] += __shfl_xor(acc[k], 32, 64);
+    }
+    if (lane < 16) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            red[wave][l16 * 8 + k] = acc[k];
+    }
+    __syncthreads();
+    if (threadIdx.x < 128) {
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < 16; ++w)
+            s += red[w][threadIdx.x];
+        out[static_cast<size_t>(h) * o_stride + threadIdx.x] = float_to_half_bits(s);
+    }
+}
+
 // One workgroup adds up 64 consecutive outputs: wavefront w takes the splits w, w + 16, ... (one
 // coalesced 256-byte row of partials each, independent loads), then the 16 wavefront sums are
 // added in wavefront order (fixed association: deterministic).
@@ -354,7 +414,11 @@ int llama2_vec_mat(llama2_half* output, const llama2_half* vector, const llama2_
     L2_CHECK(m_col_stride >= 0 && m_row_stride >= 0 && o_stride >= 0, "%s: negative stride", fn);
     const bool fast =
         rows % 8 == 0 && m_col_stride % 8 == 0 && m_row_stride % 8 == 0 && aligned(matrix, 16);
-    if (fast) {
+    if (fast && rows == 128 && cols <= kHeadVecMatCols) {
+        hipLaunchKernelGGL(vecmat_head_kernel, dim3(n_heads), dim3(1024), 0, ctx().stream, output, vector, matrix, cols,
+                           m_col_stride, o_stride, m_row_stride);
+        L2_LAUNCH_CHECK(fn);
+    } else if (fast) {
         const int hq = ceil_div(n_heads, 4), rb = ceil_div(rows, 128);
         const int t_per_wg = pick_t_per_wg(cols, hq * rb, 32);
         const int splits = ceil_div(cols, t_per_wg);

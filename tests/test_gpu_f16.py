@@ -68,7 +68,8 @@ class TestMatVecStrided:
         assert ulp_diff(actual, expected).max() <= 1
 
     @pytest.mark.parametrize("dim,heads,seq", [(4096, 32, 512), (4096, 32, 2048), (4096, 32, 4096),
-                                               (5120, 40, 777), (4096, 32, 1), (512, 2, 33)])
+                                               (5120, 40, 777), (4096, 32, 1), (512, 2, 33), (4096, 32, 100), (4096, 32, 511),
+                                               (4096, 32, 513), (5120, 40, 383)])
     def test_vs_fp64(self, oracle, dim, heads, seq):
         rng = synth.rng_for(212, dim, seq)
         hs = dim // heads
@@ -108,7 +109,8 @@ class TestVecMat:
         assert ulp_diff(actual, expected).max() <= 1
 
     @pytest.mark.parametrize("dim,heads,seq", [(4096, 32, 512), (4096, 32, 2048), (4096, 32, 4096),
-                                               (5120, 40, 777), (4096, 32, 1), (512, 2, 33)])
+                                               (5120, 40, 777), (4096, 32, 1), (512, 2, 33), (4096, 32, 100), (4096, 32, 511),
+                                               (4096, 32, 513), (5120, 40, 383)])
     def test_vs_fp64(self, oracle, dim, heads, seq):
         rng = synth.rng_for(222, dim, seq)
         hs = dim // heads
