@@ -212,6 +212,35 @@ def test_device_resident_loop_crosses_attention_shapes(oracle, mode):
         assert np.array_equal(runs[0][1].view(np.uint16), runs[1][1].view(np.uint16)), start
 
 
+def test_device_resident_loop_over_a_whole_context(oracle):
+    """4095 steps in one call: the graph replay walks through every attention launch shape (1 ... 32 blocks
+    of 128 rows, then 512-row blocks) and must produce the tokens of the same launches issued one by one;
+    the last step is checked against the module sequence on the same history."""
+    cfg = dict(HS128, n_layers=2, seq_len=4096)
+    dim, L, S = cfg["dim"], cfg["n_layers"], cfg["seq_len"]
+    model = synth.random_model(cfg, seed=13)
+    prompt = synth.rng_for(410).integers(3, cfg["vocab_size"], 6).astype(np.int32)
+    runs = []
+    for mode in (FUSED, FUSED_GRAPH):
+        t = Transformer(dict(cfg), model, mode=mode)
+        t.runstate.tokens.copy_to_device(prompt)
+        capi.call("llama2_decode_run", t._decoder, 0, S - 1, len(prompt))
+        runs.append((t.runstate.tokens.to_host(), t.runstate.logits.to_host(), t))
+    assert np.array_equal(runs[0][0], runs[1][0])
+    assert np.array_equal(runs[0][1].view(np.uint16), runs[1][1].view(np.uint16))
+    assert len(set(runs[0][0][len(prompt):].tolist())) > 50  # it decodes, it is not stuck on one token
+    t = runs[1][2]
+    m = Transformer(dict(cfg), model, mode=capi.DECODE_MODULES)
+    m.runstate.keyCache.copy_to_device(t.runstate.keyCache.to_host())
+    m.runstate.valueCache.copy_to_device(t.runstate.valueCache.to_host())
+    m.runstate.tokens.copy_to_device(runs[1][0])
+    m.Forward(S - 2, S - 1)
+    assert_close_normwise(runs[1][1], m.runstate.logits.to_host().astype(np.float64), "graph loop vs modules", 2e-3)
+    for r in runs:
+        r[2].close()
+    m.close()
+
+
 def test_generate_matches_stepwise(oracle):
     model = synth.random_model(SMALL, seed=6)
     rng = synth.rng_for(402)
