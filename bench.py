@@ -310,6 +310,15 @@ def main():
                             "pct_of_hbm_peak": round(100 * bytes_tok * tok_s / 1e9 / HBM_PEAK_GBPS, 2),
                             "bandwidth_bound_tokens_per_s": round(HBM_PEAK_GBPS * 1e9 / bytes_tok, 1),
                             "last_tokens": [int(t) for t in toks[-4:]]}
+        # the same loop late in the context: 64 steps from position 3968 of 4096 (attention reads ~2 x 1 GB of cache)
+        far = cfg["seq_len"] - 128
+        capi.call("llama2_decode_run", model._decoder, far, 8, 0)
+        capi.call("llama2_sync")
+        ev.start()
+        capi.call("llama2_decode_run", model._decoder, far, 64, 0)
+        far_ms = ev.stop_ms()
+        result["decode"]["tokens_per_s_at_position_%d" % far] = round(64 / (far_ms * 1e-3), 1)
+        log("decode at positions %d..%d: %.1f tok/s" % (far, far + 63, 64 / (far_ms * 1e-3)))
         # the reference's own loop shape (Transformer.Generate: forward, sample, read the token back on the
         # host every step) over the same launches: what a host that keeps its loop gets
         t1 = time.perf_counter()
