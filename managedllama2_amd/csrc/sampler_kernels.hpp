@@ -733,6 +733,10 @@ __device__ __noinline__ void softmax_logits_call(uint16_t* logits, int size, flo
 {
     softmax_logits_dev<CH>(logits, size, temperature, indices, *lds);
 }
+// TAG: one copy per calling kernel.  Shared between two kernels of a translation unit the same code
+// was compiled with 4.4 KB of scratch memory per lane (against 0.4 KB), and a kernel with that
+// much scratch costs over a millisecond per launch.
+template <bool TAG>
 __device__ __noinline__ void sort_lds_identity_call(uint16_t* keys, int* values, int size, SamplerLds* lds, SortLds* buf)
 {
     sort_lds_dev<true>(keys, values, size, *lds, *buf);
@@ -769,7 +773,7 @@ __device__ __forceinline__ int sample_dev(uint16_t* logits, int* indices, int si
         if (head)
             n = head;
         else if (LDS_SORT)
-            sort_lds_identity_call(logits, indices, size, &lds, buf); // indices are 0..size-1 here
+            sort_lds_identity_call<HEAD_ONLY>(logits, indices, size, &lds, buf); // indices are 0..size-1 here
         else
             sort_call<CH>(logits, indices, size, keys2, values2, &lds);
         threshold = coin * top_p;
