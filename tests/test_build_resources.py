@@ -2,7 +2,7 @@
 kilobytes per lane still computes the right thing, so no parity test notices, but every launch
 then pays for a scratch allocation of its own (measured: 1.7 ms instead of 70 us for the
 one-launch sampler).  The sampler's phases are non-inlined calls precisely to keep the register
-allocator from spilling; this compiles the two translation units that hold them and reads the
+allocator from spilling; this compiles every translation unit of the library and reads the
 compiler's own resource report."""
 import os
 import re
@@ -17,7 +17,7 @@ LIMIT = 1024  # bytes of scratch per lane
 
 
 @pytest.mark.skipif(shutil.which(HIPCC) is None, reason="hipcc not found")
-@pytest.mark.parametrize("source", ["sampler.hip", "decode.hip"])
+@pytest.mark.parametrize("source", sorted(f for f in os.listdir(CSRC) if f.endswith(".hip")))
 def test_no_kernel_needs_kilobytes_of_scratch(source, tmp_path):
     cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang",
            "-packed-fp32-ops", "-Rpass-analysis=kernel-resource-usage", "--cuda-device-only", "-c", source, "-o",
