@@ -372,12 +372,20 @@ def main():
         sampler["decode_tokens_per_s"] = round(steps / (ms * 1e-3), 1)
         sampler["decode_ms_per_token"] = round(ms / steps, 4)
         sampler["temperature"], sampler["top_p"] = temp, top_p
+        # the reference's loop shape with its sampler: forward, llama2_decode_sample_top_p, token read back per step
+        if model._decoder is not None:
+            sp, coins = model.sampler, np.random.default_rng(7)
+            sp.temperature, sp.topP, sp.random = temp, top_p, coins.random
+            t1 = time.perf_counter()
+            n_host = sum(1 for _ in model.Generate(prompt, 192, stop_on_special=False))
+            sampler["host_loop_tokens_per_s"] = round(n_host / (time.perf_counter() - t1), 1)
+            sp.temperature = 0.0
         result["sampler"] = sampler
         log("sampler (32000 logits, T=0.5, top-p 0.9): softmax %.1f + sort %.1f + cumsum %.1f + pick %.1f us; "
-            "4 launches %.1f us, one launch %.1f us; sampled decode %.1f tok/s" %
+            "4 launches %.1f us, one launch %.1f us; sampled decode %.1f tok/s (host loop %s)" %
             (sampler["softmax_logits_us"], sampler["sort_us"], sampler["cumulative_sum_us"],
              sampler["sample_top_p_us"], sampler["four_modules_us"], sampler["one_launch_us"],
-             sampler["decode_tokens_per_s"]))
+             sampler["decode_tokens_per_s"], sampler.get("host_loop_tokens_per_s")))
 
     if "repack" in legs:
         # the converter's repack of the 7B weight tensors (AWQ GEMM words -> output-major words):
