@@ -278,6 +278,41 @@ def test_llama13b_shaped_layers(oracle, mode):
     assert exact >= len(gen) - 1
 
 
+def test_decoder_create_destroy_gives_the_memory_back():
+    """A decoder owns its state block, the attention partials and up to three kinds of captured graphs per
+    attention launch shape; creating, using and destroying it repeatedly must not eat device memory."""
+    import ctypes as C
+    cfg = dict(HS128, seq_len=4096, n_layers=2)
+    model = synth.random_model(cfg, seed=14)
+    t = Transformer(dict(cfg), model, mode=None)  # owns the weights and the run state
+    w, s = t.weights.struct(), t.runstate.struct()
+    c = capi.Config(*[cfg[k] for k in ("dim", "hidden_dim", "n_layers", "n_heads", "n_kv_heads", "vocab_size", "seq_len")],
+                    cfg["rope_theta"])
+    t.runstate.tokens.copy_to_device(np.array([5, 6, 7], np.int32))
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        capi.call("llama2_mem_info", C.byref(free), C.byref(total))
+        return free.value
+
+    def cycle():
+        h = C.c_void_p()
+        capi.call("llama2_decode_create", C.byref(h), C.byref(c), C.byref(w), C.byref(s), FUSED_GRAPH)
+        capi.call("llama2_decode_run", h, 0, 6, 3)
+        capi.call("llama2_decode_run_sampled", h, 6, 4, 3, 0.7, 0.9, 1)
+        capi.call("llama2_decode_run_sampled", h, 10, 4, 3, 0.8, 0.9, 2)  # drops and rebuilds the sampled graphs
+        capi.call("llama2_decode_destroy", h)
+
+    for _ in range(3):
+        cycle()  # first uses may grow library-owned scratch
+    before = free_bytes()
+    for _ in range(40):
+        cycle()
+    capi.call("llama2_sync")
+    assert before - free_bytes() < 16 << 20, (before, free_bytes())
+    t.close()
+
+
 def test_decoder_rejects_what_the_reference_rejects():
     import ctypes as C
     model = synth.random_model(SMALL, seed=5)
