@@ -10,8 +10,10 @@
 //                          RMSNorm + SwiGLU | down-proj + residual.  Everything
 //                          that depends on the position is read from a small
 //                          device-resident state block, so the launch sequence
-//                          is identical for every token and can be replayed as
-//                          one hipGraph (LLAMA2_DECODE_GRAPH).
+//                          is identical for every token and is replayed as a
+//                          hipGraph (LLAMA2_DECODE_GRAPH): one graph per size of
+//                          the attention grid, chosen by the host's copy of the
+//                          position.
 #include "int4_kernels.hpp"
 #include "sampler_kernels.hpp"
 
