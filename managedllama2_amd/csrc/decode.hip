@@ -41,6 +41,9 @@ namespace l2 {
 // microseconds per launch at short lengths.  The position lives on the device,
 // but the host always knows an upper bound for it, so it picks the launch
 // shape (block size, number of blocks) from a short list by that bound.
+// Measured in the decode loop: one 256-row block of 8 wavefronts for 129 .. 256 rows
+// is as fast as two 128-row blocks and a merge, two 256-row blocks for 257 .. 512 rows
+// lose 1.2 % against four 128-row blocks.
 constexpr int kAttnWaves = 16;
 constexpr int kSplitT = 32 * kAttnWaves; // 512
 constexpr int kSmallWaves = 4;
@@ -71,6 +74,9 @@ inline AttnShape attn_shape(int index, int seq_len)
         return AttnShape{kAttnWaves, attn_max_splits(seq_len)};
     return AttnShape{kSmallWaves, 1 << index};
 }
+
+struct AttnArgs;
+void launch_attn(const AttnShape& shape, int n_heads, const AttnArgs& a);
 
 struct AttnArgs {
     const uint16_t* q;
@@ -238,6 +244,15 @@ __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
         }
         out[threadIdx.x] = float_to_half_bits(O / lsh[0]);
     }
+}
+
+void launch_attn(const AttnShape& shape, int n_heads, const AttnArgs& a)
+{
+    const dim3 grid(shape.splits, n_heads), block(shape.waves * 64);
+    if (shape.waves == kSmallWaves)
+        hipLaunchKernelGGL(fused_attn_kernel<kSmallWaves>, grid, block, 0, ctx().stream, a);
+    else
+        hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, grid, block, 0, ctx().stream, a);
 }
 
 // ---------------------------------------------------------------- step state
@@ -451,12 +466,7 @@ int forward_fused(llama2_decoder* d, int shape)
             a.part = d->attn_part, a.counters = d->counters, a.pos_ptr = d->state;
             a.dim = dim, a.max_splits = as.splits;
             a.scale = 1.0f / sqrtf(static_cast<float>(d->head_size));
-            if (as.waves == kSmallWaves)
-                hipLaunchKernelGGL(fused_attn_kernel<kSmallWaves>, dim3(as.splits, c.n_heads), dim3(kSmallWaves * 64), 0,
-                                   ctx().stream, a);
-            else
-                hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(as.splits, c.n_heads), dim3(kAttnWaves * 64),
-                                   0, ctx().stream, a);
+            launch_attn(as, c.n_heads, a);
             L2_LAUNCH_CHECK("fused attention");
         }
         {
@@ -613,24 +623,17 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
     L2_CHECK(n_heads <= kMaxAttnHeads, "%s: n_heads=%d exceeds %d", fn, n_heads, kMaxAttnHeads);
     L2_CHECK((static_cast<long long>(seq_length) + kSplitT) * dim * 2 < (1ll << 31),
              "%s: seq_length * dim = %lld is too large", fn, static_cast<long long>(seq_length) * dim);
-    // The caller knows the length here (the decode step does not: its position lives on the device), so
-    // the block can be matched to it: 4-wavefront workgroups over 128-row blocks spread a short
-    // sequence over more compute units, 16-wavefront workgroups over 512-row blocks need fewer merges.
-    const bool small_blocks = seq_length <= kSmallBlockMaxSeq;
-    const int block_t = small_blocks ? kSmallSplitT : kSplitT;
-    const int splits = ceil_div(seq_length, block_t);
-    L2_CHECK(splits <= kMaxSplits, "%s: seq_length=%d exceeds %d", fn, seq_length, kMaxSplits * kSplitT);
-    if (splits > 1)
-        L2_TRY(ensure_attn_partials(sizeof(float) * static_cast<size_t>(n_heads) * splits * kPartStride));
+    // The shape the decode step would pick for this length, with exactly the blocks it needs.
+    L2_CHECK(seq_length <= kMaxSplits * kSplitT, "%s: seq_length=%d exceeds %d", fn, seq_length, kMaxSplits * kSplitT);
+    AttnShape shape = attn_shape(attn_shape_index(seq_length), seq_length);
+    shape.splits = ceil_div(seq_length, shape.waves * 32);
+    if (shape.splits > 1)
+        L2_TRY(ensure_attn_partials(sizeof(float) * static_cast<size_t>(n_heads) * shape.splits * kPartStride));
     AttnArgs a{};
     a.q = query, a.kcache = key, a.vcache = value, a.out = output;
     a.part = ctx().attn_partials, a.counters = ctx().attn_counters, a.pos_ptr = nullptr, a.seq = seq_length;
-    a.dim = dim, a.max_splits = splits, a.scale = scale;
-    if (small_blocks)
-        hipLaunchKernelGGL(fused_attn_kernel<kSmallWaves>, dim3(splits, n_heads), dim3(kSmallWaves * 64), 0, ctx().stream,
-                           a);
-    else
-        hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, dim3(splits, n_heads), dim3(kAttnWaves * 64), 0, ctx().stream, a);
+    a.dim = dim, a.max_splits = shape.splits, a.scale = scale;
+    launch_attn(shape, n_heads, a);
     L2_LAUNCH_CHECK(fn);
     return LLAMA2_OK;
 }
