@@ -356,7 +356,10 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
 int llama2_decode_forward(llama2_decoder* decoder, int position, int next_position);
 /* Sampler.Sample greedy branch (src/Sampler.cs:44-47,69): argmax into
  * tokens[next_position] iff generate_token, then reads that token back
- * (the one host synchronisation per token). */
+ * (the one host synchronisation per token).  The token after the last row of
+ * the context (next_position == seq_len) has no slot in `tokens`
+ * (src/RunState.cs:52): it is returned without being stored, and the
+ * device-resident loops below do not store it either. */
 int llama2_decode_sample(llama2_decoder* decoder, int next_position, int generate_token,
                          int* token);
 /* Sampler.Sample with temperature and top-p (src/Sampler.cs:40-70): the greedy

@@ -257,10 +257,13 @@ void launch_attn(const AttnShape& shape, int n_heads, const AttnArgs& a)
 
 // ---------------------------------------------------------------- step state
 // state[0] = position, state[1] = first position whose token is generated,
-// state[2] = 1 to advance the position after sampling; the 128 floats behind
-// the 4 ints hold (cos, sin) of the position's RoPE angles, so the 32 QKV
-// launches of a step do not each spend a microsecond in powf/sinf/cosf.
-constexpr int kStateInts = 4;
+// state[2] = 1 to advance the position after sampling, state[3] = number of
+// token slots (the context length: the token after the last row has no slot and
+// is not stored), state[4] = a spare slot for that token when the host asks for
+// it; the 128 floats behind the 8 ints hold (cos, sin) of the position's RoPE
+// angles, so the 32 QKV launches of a step do not each call powf/cosf/sinf.
+constexpr int kStateInts = 8;
+constexpr int kSpareTokenSlot = 4;
 constexpr size_t kStateBytes = kStateInts * sizeof(int) + kRopeHeadSize * sizeof(float);
 
 __device__ __forceinline__ void write_rope_table(int* state, int i, int pos, float theta)
@@ -272,12 +275,13 @@ __device__ __forceinline__ void write_rope_table(int* state, int i, int pos, flo
     tab[2 * i + 1] = s;
 }
 
-__global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance, float theta)
+__global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance, int n_slots, float theta)
 {
     if (threadIdx.x == 0) {
         state[0] = pos;
         state[1] = n_prompt;
         state[2] = advance;
+        state[3] = n_slots;
     }
     if (threadIdx.x < kRopeHeadSize / 2)
         write_rope_table(state, threadIdx.x, pos, theta);
@@ -290,12 +294,13 @@ __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, in
 {
     __shared__ float sv[16];
     __shared__ int si[16];
-    const int pos0 = state[0], advance0 = state[2]; // read by every thread before thread 0 updates them
+    // read by every thread before thread 0 updates the position (one 16-byte scalar load)
+    const int pos0 = state[0], n_prompt = state[1], advance0 = state[2], n_slots = state[3];
     if (advance0 && threadIdx.x >= 64 && threadIdx.x < 64 + kRopeHeadSize / 2)
         write_rope_table(state, threadIdx.x - 64, pos0 + 1, theta); // for the next step
     const int best = block1024_argmax(x, size, sv, si);
     if (threadIdx.x == 0) {
-        if (pos0 + 1 >= state[1])
+        if (pos0 + 1 >= n_prompt && pos0 + 1 < n_slots)
             tokens[pos0 + 1] = best;
         if (advance0)
             state[0] = pos0 + 1;
@@ -321,10 +326,10 @@ struct SampleStepArgs {
 template <bool LDS_SORT>
 __device__ __forceinline__ void sample_step(const SampleStepArgs& a, SamplerLds& lds, SortLds* buf)
 {
-    const int pos0 = a.state[0], n_prompt = a.state[1], advance0 = a.state[2];
+    const int pos0 = a.state[0], n_prompt = a.state[1], advance0 = a.state[2], n_slots = a.state[3];
     if (advance0 && threadIdx.x >= 64 && threadIdx.x < 64 + kRopeHeadSize / 2)
         write_rope_table(a.state, threadIdx.x - 64, pos0 + 1, a.theta); // for the next step
-    if (pos0 + 1 >= n_prompt) { // uniform over the workgroup
+    if (pos0 + 1 >= n_prompt && pos0 + 1 < n_slots) { // uniform over the workgroup
         const float coin = sampler_coin(a.seed, pos0 + 1);
         const int token = sample_dev<LDS_SORT ? 4 : 8, LDS_SORT, true>(a.logits, a.indices, a.size, a.temperature, a.top_p,
                                                                  coin, a.keys2, a.values2, lds, buf);
@@ -525,10 +530,24 @@ int check_sampling(const char* fn, const llama2_decoder* d, float temperature)
     return LLAMA2_OK;
 }
 
+// Where the token of `next_position` goes: its slot of the run state's tokens, or, for the token
+// after the last row of the context (the reference's tokens buffer has no slot for it,
+// src/RunState.cs:52), a spare slot of the decoder's own.
+struct TokenSlot {
+    int* tokens;
+    int index;
+};
+TokenSlot token_slot(llama2_decoder* d, int next_position)
+{
+    if (next_position < d->cfg.seq_len)
+        return TokenSlot{d->s.tokens, next_position};
+    return TokenSlot{d->state, kSpareTokenSlot};
+}
+
 int set_state(llama2_decoder* d, int pos, int n_prompt, int advance)
 {
     hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, ctx().stream, d->state, pos, n_prompt, advance,
-                       d->cfg.rope_theta);
+                       d->cfg.seq_len, d->cfg.rope_theta);
     L2_LAUNCH_CHECK("set_state_kernel");
     return LLAMA2_OK;
 }
@@ -711,17 +730,24 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     d->mode = mode;
     d->kv_dim = kv_dim;
     d->head_size = c.dim / c.n_heads;
-    if (fused) {
+    {
         hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->state), kStateBytes);
         if (e == hipSuccess)
-            e = hipMalloc(reinterpret_cast<void**>(&d->attn_part),
+            e = hipMemsetAsync(d->state, 0, kStateBytes, ctx().stream);
+        if (e == hipSuccess)
+            e = hipStreamSynchronize(ctx().stream);
+        if (e != hipSuccess) {
+            release(d);
+            return hip_fail(e, "llama2_decode_create: state allocation");
+        }
+    }
+    if (fused) {
+        hipError_t e = hipMalloc(reinterpret_cast<void**>(&d->attn_part),
                           sizeof(float) * static_cast<size_t>(c.n_heads) * kMaxSplits * kPartStride);
         if (e == hipSuccess)
             e = hipMalloc(reinterpret_cast<void**>(&d->counters), sizeof(unsigned) * c.n_heads);
         if (e == hipSuccess)
             e = hipMemsetAsync(d->counters, 0, sizeof(unsigned) * c.n_heads, ctx().stream);
-        if (e == hipSuccess)
-            e = hipMemsetAsync(d->state, 0, kStateBytes, ctx().stream);
         if (e == hipSuccess)
             e = hipStreamSynchronize(ctx().stream);
         if (e != hipSuccess) {
@@ -765,8 +791,11 @@ int llama2_decode_sample(llama2_decoder* d, int next_position, int generate_toke
     L2_CHECK(d && token, "llama2_decode_sample: null argument");
     L2_CHECK(next_position >= 0 && next_position <= d->cfg.seq_len, "llama2_decode_sample: next_position=%d",
              next_position);
-    L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, d->s.tokens, next_position, generate_token));
-    return llama2_memcpy_d2h(token, d->s.tokens, static_cast<size_t>(next_position) * sizeof(int), sizeof(int));
+    const TokenSlot slot = token_slot(d, next_position);
+    L2_CHECK(slot.tokens == d->s.tokens || generate_token,
+             "llama2_decode_sample: next_position=%d is past the last token of the context", next_position);
+    L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, slot.tokens, slot.index, generate_token));
+    return llama2_memcpy_d2h(token, slot.tokens, static_cast<size_t>(slot.index) * sizeof(int), sizeof(int));
 }
 
 int llama2_decode_sample_top_p(llama2_decoder* d, int next_position, int generate_token, float temperature,
@@ -779,9 +808,10 @@ int llama2_decode_sample_top_p(llama2_decoder* d, int next_position, int generat
         return llama2_decode_sample(d, next_position, generate_token, token);
     L2_CHECK(next_position >= 0 && next_position <= d->cfg.seq_len, "%s: next_position=%d", fn, next_position);
     L2_TRY(check_sampling(fn, d, temperature));
-    L2_TRY(sample_launch(fn, d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p, coin, d->s.tokens,
-                         next_position, true)); // :50-66
-    return llama2_memcpy_d2h(token, d->s.tokens, static_cast<size_t>(next_position) * sizeof(int), sizeof(int)); // :69
+    const TokenSlot slot = token_slot(d, next_position);
+    L2_TRY(sample_launch(fn, d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p, coin, slot.tokens,
+                         slot.index, true)); // :50-66
+    return llama2_memcpy_d2h(token, slot.tokens, static_cast<size_t>(slot.index) * sizeof(int), sizeof(int)); // :69
 }
 
 float llama2_sampler_coin(unsigned long long seed, int position) { return sampler_coin(seed, position); }
@@ -800,7 +830,7 @@ int llama2_decode_run_sampled(llama2_decoder* d, int position, int steps, int n_
     if (!(d->mode & LLAMA2_DECODE_FUSED)) {
         for (int pos = position; pos < position + steps; ++pos) {
             L2_TRY(forward_modules(d, pos, pos + 1));
-            if (pos + 1 >= n_prompt)
+            if (pos + 1 >= n_prompt && pos + 1 < d->cfg.seq_len) // the token after the last row has no slot
                 L2_TRY(sample_launch(fn, d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p,
                                      sampler_coin(seed, pos + 1), d->s.tokens, pos + 1, true));
         }
@@ -837,7 +867,8 @@ int llama2_decode_run(llama2_decoder* d, int position, int steps, int n_prompt)
     if (!(d->mode & LLAMA2_DECODE_FUSED)) {
         for (int pos = position; pos < position + steps; ++pos) {
             L2_TRY(forward_modules(d, pos, pos + 1));
-            L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, d->s.tokens, pos + 1, pos + 1 >= n_prompt));
+            if (pos + 1 < d->cfg.seq_len) // the token after the last row has no slot
+                L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, d->s.tokens, pos + 1, pos + 1 >= n_prompt));
         }
         return LLAMA2_OK;
     }

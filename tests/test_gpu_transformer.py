@@ -278,6 +278,43 @@ def test_llama13b_shaped_layers(oracle, mode):
     assert exact >= len(gen) - 1
 
 
+@pytest.mark.parametrize("seq_len", [1, 2, 128, 129, 257])
+def test_context_filled_to_the_last_row(oracle, seq_len):
+    """Run to the end of contexts whose length sits on and next to the attention block size: the last step
+    attends seq_len rows.  Graph replay == eager launches bit for bit; the last logits agree with the module
+    sequence on the same history."""
+    cfg = dict(HS128, n_layers=2, seq_len=seq_len)
+    model = synth.random_model(cfg, seed=15)
+    prompt = synth.rng_for(411, seq_len).integers(3, cfg["vocab_size"], min(3, seq_len)).astype(np.int32)
+    outs = []
+    for mode in (FUSED, FUSED_GRAPH):
+        t = Transformer(dict(cfg), model, mode=mode)
+        t.runstate.tokens.copy_to_device(prompt)
+        capi.call("llama2_decode_run", t._decoder, 0, seq_len, len(prompt))  # the token after the last row is not stored
+        outs.append((t.runstate.tokens.to_host(), t.runstate.logits.to_host(), t))
+    assert np.array_equal(outs[0][0], outs[1][0])
+    assert np.array_equal(outs[0][1].view(np.uint16), outs[1][1].view(np.uint16))
+    t = outs[1][2]
+    m = Transformer(dict(cfg), model, mode=capi.DECODE_MODULES)
+    m.runstate.keyCache.copy_to_device(t.runstate.keyCache.to_host())
+    m.runstate.valueCache.copy_to_device(t.runstate.valueCache.to_host())
+    m.runstate.tokens.copy_to_device(outs[1][0])
+    m.Forward(seq_len - 1, seq_len)
+    assert_close_normwise(outs[1][1], m.runstate.logits.to_host().astype(np.float64), "graph loop vs modules", 2e-3)
+    assert capi.raw("llama2_decode_run", t._decoder, 1, seq_len, len(prompt)) == capi.ERR_INVALID_ARGUMENT  # one too many
+    # the token after the last row has no slot: it is returned, not stored (the neighbouring memory stays intact)
+    for tr in (t, m):
+        before = tr.runstate.tokens.to_host()
+        assert tr.Sample(seq_len, True) == int(np.argmax(tr.runstate.logits.to_host()))
+        assert np.array_equal(tr.runstate.tokens.to_host(), before)
+    m.sampler.temperature = t.sampler.temperature = 0.7
+    m.sampler.random = t.sampler.random = lambda: 0.25
+    assert 0 <= t.Sample(seq_len, True) < cfg["vocab_size"] and 0 <= m.Sample(seq_len, True) < cfg["vocab_size"]
+    for o in outs:
+        o[2].close()
+    m.close()
+
+
 def test_decoder_create_destroy_gives_the_memory_back():
     """A decoder owns its state block, the attention partials and up to three kinds of captured graphs per
     attention launch shape; creating, using and destroying it repeatedly must not eat device memory."""
