@@ -40,10 +40,17 @@ int ensure_attn_partials(size_t bytes);
 int sample_launch(const char* fn, uint16_t* logits, int* indices, int size, float temperature, float top_p, float coin,
                   int* result, int pos, bool token_only);
 
+// HIP's current device is a per-thread setting: a host thread other than the one that called
+// llama2_init (a thread-pool worker of the managed host, say) is bound to the library's device on
+// its first call.
+int bind_thread();
+
 #define L2_REQUIRE_INIT()                                                          \
     do {                                                                           \
         if (!::l2::ctx().ready)                                                    \
             return ::l2::fail(LLAMA2_ERR_NOT_INITIALIZED, "%s: llama2_init has not been called", __func__); \
+        if (int rc_bind_ = ::l2::bind_thread())                                    \
+            return rc_bind_;                                                       \
     } while (0)
 
 #define L2_CHECK(cond, ...)                                                        \

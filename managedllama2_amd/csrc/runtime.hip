@@ -48,6 +48,17 @@ int ensure_attn_partials(size_t bytes)
     return LLAMA2_OK;
 }
 
+int bind_thread()
+{
+    static thread_local int bound_device = -1;
+    const int device = ctx().device;
+    if (bound_device != device) {
+        L2_HIP(hipSetDevice(device));
+        bound_device = device;
+    }
+    return LLAMA2_OK;
+}
+
 } // namespace l2
 
 using namespace l2;

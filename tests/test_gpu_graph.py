@@ -123,3 +123,27 @@ def test_what_is_refused_during_capture():
         assert np.array_equal(x.to_host().view(np.uint8), np.full(128, 0x11, np.uint8))
         capi.call("llama2_memset", x.ptr, 0, 128)
     capi.call("llama2_graph_destroy", g)
+
+
+def test_calls_from_another_host_thread():
+    """The managed host builds its Transformer inside a worker task (examples/WebAPI/Program.cs:47-49): a
+    thread other than the one that called llama2_init must be able to use the library (one thread at a time)."""
+    import threading
+    model = synth.random_model(dict(CFG, seq_len=64), seed=54)
+    prompt = [5, 9, 11]
+    want = list(Transformer(dict(CFG, seq_len=64), model, mode=FUSED_GRAPH).Generate(prompt, 12, stop_on_special=False))
+    got, errors = [], []
+
+    def worker():
+        try:
+            t = Transformer(dict(CFG, seq_len=64), model, mode=FUSED_GRAPH)
+            got.extend(t.Generate(prompt, 12, stop_on_special=False))
+            t.close()
+        except Exception as e:  # surfaced in the main thread below
+            errors.append(e)
+
+    th = threading.Thread(target=worker)
+    th.start()
+    th.join(120)
+    assert not th.is_alive() and not errors, errors
+    assert got == want
