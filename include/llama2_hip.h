@@ -20,9 +20,10 @@
  *   - all pointers named out/x/q/... are DEVICE pointers obtained from
  *     llama2_malloc (or any hipMalloc'ed memory of the same device);
  *   - kernels are enqueued asynchronously on one library-owned stream, in
- *     call order; llama2_memcpy_d2h and llama2_sync wait for them.  Like the
- *     reference (single NULL stream, one host thread) the library is not
- *     re-entrant.
+ *     call order; llama2_memcpy_d2h and llama2_sync wait for them.  The
+ *     reference runs on a single NULL stream from one host thread; here host
+ *     threads may share the library: every entry point takes one lock and
+ *     binds the calling thread to the library's device, so calls take turns.
  */
 #ifndef LLAMA2_HIP_H
 #define LLAMA2_HIP_H

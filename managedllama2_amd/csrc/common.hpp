@@ -7,6 +7,7 @@
 #include <cstdarg>
 #include <cstddef>
 #include <cstdint>
+#include <mutex>
 
 #include "../../include/llama2_hip.h"
 
@@ -45,7 +46,14 @@ int sample_launch(const char* fn, uint16_t* logits, int* indices, int size, floa
 // its first call.
 int bind_thread();
 
+// Every entry point runs under one recursive lock (entry points call each other): host threads
+// that share the library -- one Transformer per connection, say -- take turns.  The GPU work is in
+// order on one stream either way; what the lock protects is the stream-capture state and the lazily
+// captured graphs.  llama2_graph_begin_capture keeps the lock until llama2_graph_end_capture.
+std::recursive_mutex& api_mutex();
+
 #define L2_REQUIRE_INIT()                                                          \
+    std::lock_guard<std::recursive_mutex> l2_api_lock_(::l2::api_mutex());         \
     do {                                                                           \
         if (!::l2::ctx().ready)                                                    \
             return ::l2::fail(LLAMA2_ERR_NOT_INITIALIZED, "%s: llama2_init has not been called", __func__); \

@@ -882,6 +882,7 @@ int llama2_decode_destroy(llama2_decoder* d)
 {
     if (!d)
         return LLAMA2_OK;
+    std::lock_guard<std::recursive_mutex> lock(api_mutex());
     if (ctx().ready)
         L2_HIP(hipStreamSynchronize(ctx().stream));
     release(d);

@@ -48,6 +48,12 @@ int ensure_attn_partials(size_t bytes)
     return LLAMA2_OK;
 }
 
+std::recursive_mutex& api_mutex()
+{
+    static std::recursive_mutex m;
+    return m;
+}
+
 int bind_thread()
 {
     static thread_local int bound_device = -1;
@@ -69,6 +75,7 @@ const char* llama2_last_error(void) { return g_err; }
 
 int llama2_init(int device)
 {
+    std::lock_guard<std::recursive_mutex> lock(api_mutex());
     Context& c = ctx();
     if (c.ready && c.device == device)
         return LLAMA2_OK;
@@ -100,6 +107,7 @@ int llama2_init(int device)
 
 int llama2_shutdown(void)
 {
+    std::lock_guard<std::recursive_mutex> lock(api_mutex());
     Context& c = ctx();
     if (!c.ready)
         return LLAMA2_OK;
@@ -265,6 +273,7 @@ int llama2_graph_begin_capture(void)
     L2_NOT_CAPTURING("llama2_graph_begin_capture");
     L2_HIP(hipStreamBeginCapture(ctx().stream, hipStreamCaptureModeThreadLocal));
     ctx().capturing = true;
+    api_mutex().lock(); // released by llama2_graph_end_capture: no other thread may launch into the capture
     return LLAMA2_OK;
 }
 
@@ -277,7 +286,10 @@ int llama2_graph_end_capture(void** graph)
         return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_graph_end_capture: no capture in progress");
     ctx().capturing = false;
     hipGraph_t g = nullptr;
-    L2_HIP(hipStreamEndCapture(ctx().stream, &g));
+    const hipError_t ended = hipStreamEndCapture(ctx().stream, &g);
+    api_mutex().unlock(); // taken by llama2_graph_begin_capture (this call still holds its own)
+    if (ended != hipSuccess)
+        return hip_fail(ended, "hipStreamEndCapture");
     hipGraphExec_t exec = nullptr;
     hipError_t e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
     (void)hipGraphDestroy(g);

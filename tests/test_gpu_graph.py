@@ -147,3 +147,36 @@ def test_calls_from_another_host_thread():
     th.join(120)
     assert not th.is_alive() and not errors, errors
     assert got == want
+
+
+def test_sessions_on_concurrent_host_threads():
+    """One Transformer per connection on thread-pool threads (examples/WebSocket/Program.cs:85): the entry
+    points take turns under the library's lock, so concurrent sessions produce what each produces alone,
+    including decoders created (which captures graphs) while another session is decoding."""
+    import threading
+    cfg = dict(CFG, seq_len=96)
+    model = synth.random_model(cfg, seed=55)
+    prompts = [[5, 9, 11], [7, 8], [100, 200, 300, 400], [3, 4, 5]]
+    want = []
+    for p in prompts:
+        t = Transformer(dict(cfg), model, mode=FUSED_GRAPH)
+        want.append(list(t.Generate(p, 40, stop_on_special=False)))
+        t.close()
+    got, errors = [None] * len(prompts), []
+
+    def worker(i):
+        try:
+            for _ in range(3):  # create / decode / destroy repeatedly while the others run
+                t = Transformer(dict(cfg), model, mode=FUSED_GRAPH if i % 2 == 0 else FUSED)
+                got[i] = list(t.Generate(prompts[i], 40, stop_on_special=False))
+                t.close()
+        except Exception as e:
+            errors.append((i, e))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(prompts))]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join(180)
+    assert not any(th.is_alive() for th in threads) and not errors, errors
+    assert got == want
