@@ -46,6 +46,7 @@ typedef uint16_t llama2_half;
 #define LLAMA2_ERR_NOT_INITIALIZED (-2)  /* llama2_init not called                        */
 #define LLAMA2_ERR_UNSUPPORTED (-3)      /* shape outside what the kernels implement      */
 #define LLAMA2_ERR_NO_DEVICE (-4)        /* no usable gfx950 device                        */
+#define LLAMA2_ERR_STEP_FAILED (-5)      /* a persistent decode step gave up a bounded wait */
 
 /* Largest softmax row, as in the reference (native/softmax_kernel.cu:5). */
 #define LLAMA2_MAX_SOFTMAX_SIZE 8192
@@ -96,9 +97,12 @@ int llama2_event_destroy(void* event);
  * llama2_graph_launch replays with a single submission (no counterpart in the
  * reference, which pays one cuLaunchKernel per module call, src/Module.cs:21-22).
  * Only kernel entry points may be called while capturing: no malloc / free /
- * memcpy / sync, and llama2_vec_mat only for shapes whose scratch already
- * exists (call it once eagerly first).  The captured calls keep the argument
- * values they were made with. */
+ * memcpy / sync, and llama2_vec_mat / llama2_multi_head_attention only for
+ * shapes whose scratch already exists (call them once eagerly first, or use
+ * llama2_multi_head_attention_static).  The captured calls keep the argument
+ * values they were made with, the scratch address included: the library never
+ * frees a scratch buffer before llama2_shutdown, so a later eager call that
+ * needs a larger one leaves earlier graphs valid. */
 int llama2_graph_begin_capture(void);
 int llama2_graph_end_capture(void** graph);
 int llama2_graph_launch(void* graph);
@@ -190,6 +194,24 @@ int llama2_vec_mat(llama2_half* output, const llama2_half* vector, const llama2_
 int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, const llama2_half* key,
                                 const llama2_half* value, int head_size, int dim, int seq_length,
                                 float scale, int n_heads);
+
+/* llama2_multi_head_attention for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  Same arguments, same
+ * kernels and bit-identical results; the partial results of the blocks a long
+ * sequence is split into go to a fixed array inside the library (about 2.1 MB
+ * per GPU, held until the process ends) instead of a buffer that grows on
+ * demand, so the call never allocates or frees.  Limit: n_heads times the
+ * number of blocks (128 rows each up to 3072 rows, 512 rows beyond) must not
+ * exceed LLAMA2_STATIC_ATTENTION_BLOCKS, else LLAMA2_ERR_UNSUPPORTED.  Every
+ * call on a GPU shares that GPU's array: calls are ordered on the library's
+ * one stream; a caller that replays captured graphs of this call on streams
+ * of its own must not let two of them overlap. */
+#define LLAMA2_STATIC_ATTENTION_BLOCKS 4096
+int llama2_multi_head_attention_static(llama2_half* output, const llama2_half* query,
+                                       const llama2_half* key, const llama2_half* value,
+                                       int head_size, int dim, int seq_length, float scale,
+                                       int n_heads);
 
 /* ------------------------------------------------------- pointwise modules */
 
@@ -344,6 +366,19 @@ typedef struct llama2_decoder llama2_decoder;
 #define LLAMA2_DECODE_MODULES 0 /* the 10 module launches per layer of Transformer.Forward */
 #define LLAMA2_DECODE_FUSED 1   /* fused kernels (norm+QKV+RoPE, attention, norm+SwiGLU, ...) */
 #define LLAMA2_DECODE_GRAPH 2   /* OR-able: replay the step as a captured hipGraph (one per attention launch shape) */
+/* OR-able with LLAMA2_DECODE_FUSED: the whole of Transformer.Forward
+ * (src/Transformer.cs:158-190) as ONE persistent launch -- one workgroup per
+ * compute unit walks through all layers, the vectors between the modules are
+ * handed from workgroup to workgroup inside the launch, and the weight stream
+ * never stops at a module boundary.  Same arithmetic, same results as
+ * LLAMA2_DECODE_FUSED.  Serves histories of up to 3072 rows (longer ones fall
+ * back to the launch sequence, step by step) and the shapes it has kernels for
+ * (Llama-2-7B: dim 4096, hidden_dim 11008, 32 heads on 256 compute units; and
+ * models up to dim 2048 / hidden_dim 2048); otherwise llama2_decode_create
+ * returns LLAMA2_ERR_UNSUPPORTED.  The launch needs the GPU to itself: all its
+ * workgroups must be resident at once.  Every wait inside it is bounded; a step
+ * that gives up raises a flag that llama2_decode_check reports. */
+#define LLAMA2_DECODE_PERSISTENT 4
 
 /* Binds a config, a weight set and a run state (all borrowed, all must outlive
  * the decoder) to the per-step launch sequence of Transformer.Forward
@@ -390,6 +425,26 @@ int llama2_decode_run(llama2_decoder* decoder, int position, int steps, int n_pr
  * is sorted and summed. */
 int llama2_decode_run_sampled(llama2_decoder* decoder, int position, int steps, int n_prompt,
                               float temperature, float top_p, unsigned long long seed);
+/* Waits for the enqueued steps and reports LLAMA2_ERR_STEP_FAILED if a
+ * persistent step (LLAMA2_DECODE_PERSISTENT) gave up a wait; LLAMA2_OK for the
+ * other modes.  No counterpart in the reference (its kernels cannot fail this
+ * way). */
+int llama2_decode_check(llama2_decoder* decoder);
+/* Number of unsuccessful polls (about a microsecond each) after which a wait
+ * inside the persistent step gives up; default 2^21.  Clears the failure flag.
+ * For tests of the failure path and for hosts that want a tighter bound. */
+int llama2_decode_set_wait_limit(llama2_decoder* decoder, int polls);
+/* The int4 mat-vec set of every layer of the decoder's model -- RMSNorm + fused
+ * QKV (native/mat_vec_kernel.cu:166-203), o-proj + residual (:144-164), RMSNorm
+ * + fused SwiGLU (:206-234), down-proj + residual -- chained through all layers
+ * in one persistent launch, exactly as the persistent step runs them, but
+ * without attention: the o-projection takes q as its input.  input: dim halfs
+ * (the residual stream entering layer 0); output: dim halfs (the residual
+ * stream after the last layer).  Needs LLAMA2_DECODE_PERSISTENT.  This is the
+ * measurement and parity handle for the mat-vec family inside the persistent
+ * step; the KV cache is not touched. */
+int llama2_decode_matvec_chain(llama2_decoder* decoder, const llama2_half* input,
+                               llama2_half* output);
 int llama2_decode_destroy(llama2_decoder* decoder);
 
 #if defined(__GNUC__)

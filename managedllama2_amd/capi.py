@@ -13,12 +13,15 @@ ERR_INVALID_ARGUMENT = -1
 ERR_NOT_INITIALIZED = -2
 ERR_UNSUPPORTED = -3
 ERR_NO_DEVICE = -4
+ERR_STEP_FAILED = -5
 MAX_SOFTMAX_SIZE = 8192
 MAX_SAMPLER_SIZE = 65536
+STATIC_ATTENTION_BLOCKS = 4096
 
 DECODE_MODULES = 0
 DECODE_FUSED = 1
 DECODE_GRAPH = 2
+DECODE_PERSISTENT = 4
 
 vp = C.c_void_p
 i = C.c_int
@@ -92,6 +95,7 @@ _SIGNATURES = {
     "llama2_mat_vec_strided": [vp, vp, vp, i, i, i, i, i, i, f, i],
     "llama2_vec_mat": [vp, vp, vp, i, i, i, i, i, i],
     "llama2_multi_head_attention": [vp, vp, vp, vp, i, i, i, f, i],
+    "llama2_multi_head_attention_static": [vp, vp, vp, vp, i, i, i, f, i],
     "llama2_rmsnorm": [vp, vp, vp, i, f],
     "llama2_rope": [vp, vp, i, i, i, f, i],
     "llama2_softmax": [vp, i, i],
@@ -112,6 +116,9 @@ _SIGNATURES = {
     "llama2_decode_sample_top_p": [vp, i, i, f, f, f, C.POINTER(i)],
     "llama2_decode_run": [vp, i, i, i],
     "llama2_decode_run_sampled": [vp, i, i, i, f, f, C.c_ulonglong],
+    "llama2_decode_check": [vp],
+    "llama2_decode_set_wait_limit": [vp, i],
+    "llama2_decode_matvec_chain": [vp, vp, vp],
     "llama2_decode_destroy": [vp],
 }
 # exported, not status-returning

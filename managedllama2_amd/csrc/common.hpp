@@ -14,6 +14,8 @@
 namespace l2 {
 
 // ------------------------------------------------------------------ host side
+constexpr int kMaxRetiredPartials = 32;
+
 struct Context {
     bool ready = false;
     int device = -1;
@@ -23,6 +25,10 @@ struct Context {
     // fp32 partial sums of the sequence-split attention kernels
     float* attn_partials = nullptr;
     size_t attn_partials_bytes = 0;
+    // earlier, smaller buffers: a graph captured by the caller may still hold their address,
+    // so they stay allocated until llama2_shutdown
+    float* retired_partials[kMaxRetiredPartials] = {};
+    int n_retired_partials = 0;
     // per-head arrival counters of llama2_multi_head_attention (zero between launches)
     unsigned* attn_counters = nullptr;
     // second buffer of the sampler's radix sort (LLAMA2_MAX_SAMPLER_SIZE keys and payloads)
@@ -36,6 +42,9 @@ Context& ctx();
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char* what);
 int ensure_attn_partials(size_t bytes);
+// Resolves the device address of the file-scope scratch of llama2_multi_head_attention_static
+// (decode.hip) for `device`, which must be current; called once per device by llama2_init.
+int resolve_static_scratch(int device);
 // Sampler.Sample's stochastic branch in one launch (sampler.hip).  token_only: the caller reads the
 // token alone, so the sort may stop at the head of the distribution that holds top_p of the mass.
 int sample_launch(const char* fn, uint16_t* logits, int* indices, int size, float temperature, float top_p, float coin,

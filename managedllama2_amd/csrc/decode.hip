@@ -15,6 +15,7 @@
 //                          the attention grid, chosen by the host's copy of the
 //                          position.
 #include "int4_kernels.hpp"
+#include "persist.hpp"
 #include "sampler_kernels.hpp"
 
 #include <climits>
@@ -260,10 +261,11 @@ void launch_attn(const AttnShape& shape, int n_heads, const AttnArgs& a)
 // state[2] = 1 to advance the position after sampling, state[3] = number of
 // token slots (the context length: the token after the last row has no slot and
 // is not stored), state[4] = a spare slot for that token when the host asks for
-// it; the 128 floats behind the 8 ints hold (cos, sin) of the position's RoPE
+// it, state[5] = a serial number that every kernel which sets or advances the
+// position increments (the persistent step derives its hand-over tags from it),
+// state[6] = the persistent step's error flag (persist.hpp names the indices);
+// the 128 floats behind the 8 ints hold (cos, sin) of the position's RoPE
 // angles, so the 32 QKV launches of a step do not each call powf/cosf/sinf.
-constexpr int kStateInts = 8;
-constexpr int kSpareTokenSlot = 4;
 constexpr size_t kStateBytes = kStateInts * sizeof(int) + kRopeHeadSize * sizeof(float);
 
 __device__ __forceinline__ void write_rope_table(int* state, int i, int pos, float theta)
@@ -282,9 +284,16 @@ __global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance,
         state[1] = n_prompt;
         state[2] = advance;
         state[3] = n_slots;
+        state[kStateSerial] = state[kStateSerial] + 1;
     }
     if (threadIdx.x < kRopeHeadSize / 2)
         write_rope_table(state, threadIdx.x, pos, theta);
+}
+
+__global__ void bump_serial_kernel(int* state)
+{
+    if (threadIdx.x == 0)
+        state[kStateSerial] = state[kStateSerial] + 1;
 }
 
 // Sampler.Sample greedy branch (src/Sampler.cs:44-47) against the device state:
@@ -304,6 +313,7 @@ __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, in
             tokens[pos0 + 1] = best;
         if (advance0)
             state[0] = pos0 + 1;
+        state[kStateSerial] = state[kStateSerial] + 1;
     }
 }
 
@@ -337,8 +347,11 @@ __device__ __forceinline__ void sample_step(const SampleStepArgs& a, SamplerLds&
             a.tokens[pos0 + 1] = token;
     }
     __syncthreads(); // every thread has read the state
-    if (threadIdx.x == 0 && advance0)
-        a.state[0] = pos0 + 1;
+    if (threadIdx.x == 0) {
+        if (advance0)
+            a.state[0] = pos0 + 1;
+        a.state[kStateSerial] = a.state[kStateSerial] + 1;
+    }
 }
 
 __global__ __launch_bounds__(kSampBlock) void sample_step_kernel(SampleStepArgs a)
@@ -372,9 +385,16 @@ struct llama2_decoder {
     // Forward + greedy sample + position advance; Forward + stochastic sample + position
     // advance, captured for the parameters below.
     enum { kGraphForward, kGraphStep, kGraphStepSampled, kGraphKinds };
-    hipGraphExec_t graphs[kGraphKinds][l2::kAttnShapes] = {};
+    // the last shape index is the persistent step (one launch for any history up to kPMaxRows rows)
+    hipGraphExec_t graphs[kGraphKinds][l2::kAttnShapes + 1] = {};
     float sampled_temperature = 0.0f, sampled_top_p = 0.0f;
     unsigned long long sampled_seed = 0;
+    // persistent step (LLAMA2_DECODE_PERSISTENT): kernel variant, per-layer pointer table and
+    // hand-over buffers on the device, and the launch arguments
+    int persist_variant = -1;
+    l2::PersistLayer* persist_layers = nullptr;
+    void* persist_scratch = nullptr;
+    l2::PersistArgs pa{};
 };
 
 using namespace l2;
@@ -438,10 +458,49 @@ int forward_modules(llama2_decoder* d, int position, int next_position)
 
 QW qw(const llama2_qweight& q) { return QW{q.weight, q.zeros, q.scales}; }
 
+constexpr int kPersistShape = kAttnShapes; // index of the persistent step among the launch shapes
+
+// Device-side tables and hand-over buffers of the persistent step.
+int persist_setup(llama2_decoder* d)
+{
+    const llama2_config& c = d->cfg;
+    std::vector<PersistLayer> table(c.n_layers);
+    for (int i = 0; i < c.n_layers; ++i) {
+        const llama2_layer_weights& L = d->layers[i];
+        table[i] = PersistLayer{qw(L.query), qw(L.key),  qw(L.value),     qw(L.output),      qw(L.gate),
+                                qw(L.up),    qw(L.down), L.rms_attention, L.rms_feed_forward};
+    }
+    const size_t table_bytes = sizeof(PersistLayer) * table.size();
+    L2_HIP(hipMalloc(reinterpret_cast<void**>(&d->persist_layers), table_bytes));
+    L2_HIP(hipMemcpyAsync(d->persist_layers, table.data(), table_bytes, hipMemcpyHostToDevice, ctx().stream));
+    const size_t scratch_bytes = persist_scratch_bytes(c.dim, c.hidden_dim, c.n_heads);
+    L2_HIP(hipMalloc(&d->persist_scratch, scratch_bytes));
+    L2_HIP(hipMemsetAsync(d->persist_scratch, 0, scratch_bytes, ctx().stream)); // tag 0: no word is ready
+    L2_HIP(hipStreamSynchronize(ctx().stream)); // `table` goes out of scope
+    PersistArgs& a = d->pa;
+    a = PersistArgs{};
+    a.layers = d->persist_layers;
+    a.n_layers = c.n_layers, a.dim = c.dim, a.hidden = c.hidden_dim, a.n_heads = c.n_heads, a.vocab = c.vocab_size;
+    a.seq_len = c.seq_len;
+    a.ss_d = ceil_div(c.dim, 128), a.ws_d = ceil_div(c.dim, 32) * 4, a.zs_d = ceil_div(a.ss_d, 8);
+    a.ss_h = ceil_div(c.hidden_dim, 128), a.ws_h = ceil_div(c.hidden_dim, 32) * 4, a.zs_h = ceil_div(a.ss_h, 8);
+    a.eps = 1e-5f;
+    a.scale = 1.0f / sqrtf(static_cast<float>(d->head_size));
+    a.embedding = d->w.token_embedding_table, a.tokens = d->s.tokens;
+    a.rms_final = d->w.rms_final_weight, a.classifier = d->w.classifier_weights, a.logits = d->s.logits;
+    a.kcache = d->s.key_cache, a.vcache = d->s.value_cache;
+    a.state = d->state;
+    a.spin_limit = kPersistSpinLimit;
+    persist_bind_scratch(a, d->persist_scratch);
+    return LLAMA2_OK;
+}
+
 // The same step in 5 launches per layer; the position comes from d->state, and
 // `shape` (attn_shape_index of an upper bound of position + 1) sizes the attention grid.
 int forward_fused(llama2_decoder* d, int shape)
 {
+    if (shape == kPersistShape) // the whole step in one launch
+        return persist_launch(d->persist_variant, d->pa, ctx().num_cus);
     const AttnShape as = attn_shape(shape, d->cfg.seq_len);
     const llama2_config& c = d->cfg;
     const llama2_run_state& s = d->s;
@@ -582,7 +641,10 @@ int capture(hipGraphExec_t* exec, llama2_decoder* d, int kind, int shape)
 // step may be replayed at any later position, so it gets the shape of the whole context.
 int step_shape(const llama2_decoder* d, int position)
 {
-    return attn_shape_index(ctx().capturing ? d->cfg.seq_len : position + 1);
+    const int rows = ctx().capturing ? d->cfg.seq_len : position + 1;
+    if (d->persist_variant >= 0 && rows <= kPMaxRows)
+        return kPersistShape;
+    return attn_shape_index(rows);
 }
 
 // Launches one step of `kind`: the captured graph of that shape (captured on first use)
@@ -613,6 +675,10 @@ void release(llama2_decoder* d)
                 (void)hipGraphExecDestroy(g);
     if (d->state)
         (void)hipFree(d->state);
+    if (d->persist_layers)
+        (void)hipFree(d->persist_layers);
+    if (d->persist_scratch)
+        (void)hipFree(d->persist_scratch);
     if (d->attn_part)
         (void)hipFree(d->attn_part);
     if (d->counters)
@@ -620,16 +686,11 @@ void release(llama2_decoder* d)
     delete d;
 }
 
-} // namespace
-
-extern "C" {
-
-int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, const llama2_half* key,
-                                const llama2_half* value, int head_size, int dim, int seq_length, float scale,
-                                int n_heads)
+// Argument checks shared by the two attention entry points; on success *shape is the launch
+// shape the decode step would pick for this length, with exactly the blocks it needs.
+int check_attention(const char* fn, const void* output, const void* query, const void* key, const void* value,
+                    int head_size, int dim, int seq_length, int n_heads, AttnShape* shape)
 {
-    L2_REQUIRE_INIT();
-    const char* fn = "llama2_multi_head_attention";
     L2_CHECK(output && query && key && value, "%s: null pointer", fn);
     L2_CHECK(seq_length > 0 && n_heads > 0 && dim > 0, "%s: seq_length=%d n_heads=%d dim=%d must be positive", fn,
              seq_length, n_heads, dim);
@@ -642,15 +703,106 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
     L2_CHECK(n_heads <= kMaxAttnHeads, "%s: n_heads=%d exceeds %d", fn, n_heads, kMaxAttnHeads);
     L2_CHECK((static_cast<long long>(seq_length) + kSplitT) * dim * 2 < (1ll << 31),
              "%s: seq_length * dim = %lld is too large", fn, static_cast<long long>(seq_length) * dim);
-    // The shape the decode step would pick for this length, with exactly the blocks it needs.
     L2_CHECK(seq_length <= kMaxSplits * kSplitT, "%s: seq_length=%d exceeds %d", fn, seq_length, kMaxSplits * kSplitT);
-    AttnShape shape = attn_shape(attn_shape_index(seq_length), seq_length);
-    shape.splits = ceil_div(seq_length, shape.waves * 32);
+    *shape = attn_shape(attn_shape_index(seq_length), seq_length);
+    shape->splits = ceil_div(seq_length, shape->waves * 32);
+    return LLAMA2_OK;
+}
+
+} // namespace
+
+// ---------------------------------------------------------------- static scratch
+// llama2_multi_head_attention_static allocates nothing: the partial results of the
+// blocks of a head and the heads' arrival counters live in this file-scope device
+// array (one copy per GPU, at its own address, for the life of the process).  In host
+// code the array's name is only a stand-in; its device address is asked for once per
+// device at llama2_init and every later use goes through that pointer.
+namespace l2 {
+struct StaticAttnScratch {
+    float part[static_cast<size_t>(LLAMA2_STATIC_ATTENTION_BLOCKS) * kPartStride];
+    unsigned counters[kMaxAttnHeads];
+};
+} // namespace l2
+static __device__ __align__(256) unsigned char scratch[sizeof(l2::StaticAttnScratch)];
+
+namespace l2 {
+constexpr int kMaxDevices = 64;
+static StaticAttnScratch* g_static_scratch[kMaxDevices] = {};
+
+static StaticAttnScratch* static_scratch_of(int device)
+{
+    return device >= 0 && device < kMaxDevices ? g_static_scratch[device] : nullptr;
+}
+
+__global__ void clear_words_kernel(unsigned* p, int n)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n)
+        p[i] = 0u;
+}
+
+// Called by llama2_init with `device` current: resolves this device's copy of the array
+// and clears the arrival counters (the kernels leave them at zero after every launch).
+int resolve_static_scratch(int device)
+{
+    if (device < 0 || device >= kMaxDevices)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_init: device %d beyond the %d the static scratch tracks", device,
+                    kMaxDevices);
+    void* ptr = nullptr;
+    L2_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr)
+        return fail(LLAMA2_ERR_NO_DEVICE, "llama2_init: the static scratch has no address on device %d", device);
+    StaticAttnScratch* sp = static_cast<StaticAttnScratch*>(ptr);
+    hipLaunchKernelGGL(clear_words_kernel, dim3(ceil_div(kMaxAttnHeads, 256)), dim3(256), 0, ctx().stream, sp->counters,
+                       kMaxAttnHeads);
+    L2_LAUNCH_CHECK("clear_words_kernel");
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    g_static_scratch[device] = sp;
+    return LLAMA2_OK;
+}
+} // namespace l2
+
+extern "C" {
+
+int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, const llama2_half* key,
+                                const llama2_half* value, int head_size, int dim, int seq_length, float scale,
+                                int n_heads)
+{
+    L2_REQUIRE_INIT();
+    const char* fn = "llama2_multi_head_attention";
+    AttnShape shape{};
+    L2_TRY(check_attention(fn, output, query, key, value, head_size, dim, seq_length, n_heads, &shape));
     if (shape.splits > 1)
         L2_TRY(ensure_attn_partials(sizeof(float) * static_cast<size_t>(n_heads) * shape.splits * kPartStride));
     AttnArgs a{};
     a.q = query, a.kcache = key, a.vcache = value, a.out = output;
     a.part = ctx().attn_partials, a.counters = ctx().attn_counters, a.pos_ptr = nullptr, a.seq = seq_length;
+    a.dim = dim, a.max_splits = shape.splits, a.scale = scale;
+    launch_attn(shape, n_heads, a);
+    L2_LAUNCH_CHECK(fn);
+    return LLAMA2_OK;
+}
+
+int llama2_multi_head_attention_static(llama2_half* output, const llama2_half* query, const llama2_half* key,
+                                       const llama2_half* value, int head_size, int dim, int seq_length,
+                                       float scale, int n_heads)
+{
+    L2_REQUIRE_INIT();
+    const char* fn = "llama2_multi_head_attention_static";
+    AttnShape shape{};
+    L2_TRY(check_attention(fn, output, query, key, value, head_size, dim, seq_length, n_heads, &shape));
+    StaticAttnScratch* sp = static_scratch_of(ctx().device);
+    if (!sp)
+        return fail(LLAMA2_ERR_NOT_INITIALIZED, "%s: the static scratch of device %d was not resolved at llama2_init", fn,
+                    ctx().device);
+    if (static_cast<long long>(n_heads) * shape.splits > LLAMA2_STATIC_ATTENTION_BLOCKS)
+        return fail(LLAMA2_ERR_UNSUPPORTED,
+                    "%s: n_heads=%d x %d blocks of %d rows exceed the static scratch of %d (head, block) pairs; "
+                    "use llama2_multi_head_attention",
+                    fn, n_heads, shape.splits, shape.waves * 32, LLAMA2_STATIC_ATTENTION_BLOCKS);
+    AttnArgs a{};
+    a.q = query, a.kcache = key, a.vcache = value, a.out = output;
+    a.part = sp->part, a.counters = sp->counters, a.pos_ptr = nullptr, a.seq = seq_length;
     a.dim = dim, a.max_splits = shape.splits, a.scale = scale;
     launch_attn(shape, n_heads, a);
     L2_LAUNCH_CHECK(fn);
@@ -679,11 +831,21 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     if (c.seq_len > LLAMA2_MAX_SOFTMAX_SIZE)
         return fail(LLAMA2_ERR_UNSUPPORTED, "%s: seq_len=%d exceeds the softmax limit %d", fn, c.seq_len,
                     LLAMA2_MAX_SOFTMAX_SIZE);
-    L2_CHECK(mode >= 0 && mode <= (LLAMA2_DECODE_FUSED | LLAMA2_DECODE_GRAPH), "%s: unknown mode %d", fn, mode);
+    L2_CHECK(mode >= 0 && mode <= (LLAMA2_DECODE_FUSED | LLAMA2_DECODE_GRAPH | LLAMA2_DECODE_PERSISTENT),
+             "%s: unknown mode %d", fn, mode);
     const bool fused = (mode & LLAMA2_DECODE_FUSED) != 0;
-    if ((mode & LLAMA2_DECODE_GRAPH) && !fused)
+    if ((mode & (LLAMA2_DECODE_GRAPH | LLAMA2_DECODE_PERSISTENT)) && !fused)
         return fail(LLAMA2_ERR_UNSUPPORTED,
-                    "%s: LLAMA2_DECODE_GRAPH needs LLAMA2_DECODE_FUSED (the module sequence takes the position by value)", fn);
+                    "%s: LLAMA2_DECODE_GRAPH and LLAMA2_DECODE_PERSISTENT need LLAMA2_DECODE_FUSED (the module sequence "
+                    "takes the position by value)", fn);
+    int variant = -1;
+    if (mode & LLAMA2_DECODE_PERSISTENT) {
+        variant = persist_variant(c.dim, c.hidden_dim, c.n_heads, ctx().num_cus);
+        if (variant < 0)
+            return fail(LLAMA2_ERR_UNSUPPORTED,
+                        "%s: no persistent step for dim %d, hidden_dim %d, %d heads on %d compute units; drop "
+                        "LLAMA2_DECODE_PERSISTENT", fn, c.dim, c.hidden_dim, c.n_heads, ctx().num_cus);
+    }
     if (fused) {
         const int head_size = c.dim / c.n_heads;
         if (head_size != kRopeHeadSize || c.dim % 8 || c.hidden_dim % 8 ||
@@ -754,9 +916,26 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
             release(d);
             return hip_fail(e, "llama2_decode_create: scratch allocation");
         }
+        if (variant >= 0) {
+            const int rc = persist_setup(d);
+            if (rc != LLAMA2_OK) {
+                release(d);
+                return rc;
+            }
+            d->persist_variant = variant;
+        }
         if (mode & LLAMA2_DECODE_GRAPH) { // every shape this context can reach, so that no step pays for a capture
             int rc = LLAMA2_OK;
-            for (int shape = 0; shape <= attn_shape_index(c.seq_len) && rc == LLAMA2_OK; ++shape) {
+            if (variant >= 0) {
+                rc = capture(&d->graphs[llama2_decoder::kGraphForward][kPersistShape], d, llama2_decoder::kGraphForward,
+                             kPersistShape);
+                if (rc == LLAMA2_OK)
+                    rc = capture(&d->graphs[llama2_decoder::kGraphStep][kPersistShape], d, llama2_decoder::kGraphStep,
+                                 kPersistShape);
+            }
+            // the launch sequence serves what the persistent step does not: histories beyond kPMaxRows rows
+            const int first = variant >= 0 ? attn_shape_index(kPMaxRows + 1) : 0;
+            for (int shape = first; shape <= attn_shape_index(c.seq_len) && rc == LLAMA2_OK; ++shape) {
                 rc = capture(&d->graphs[llama2_decoder::kGraphForward][shape], d, llama2_decoder::kGraphForward, shape);
                 if (rc == LLAMA2_OK)
                     rc = capture(&d->graphs[llama2_decoder::kGraphStep][shape], d, llama2_decoder::kGraphStep, shape);
@@ -876,6 +1055,59 @@ int llama2_decode_run(llama2_decoder* d, int position, int steps, int n_prompt)
     for (int i = 0; i < steps; ++i)
         L2_TRY(launch_step(d, llama2_decoder::kGraphStep, position + i));
     return LLAMA2_OK;
+}
+
+int llama2_decode_check(llama2_decoder* d)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(d, "llama2_decode_check: null decoder");
+    L2_CHECK(!ctx().capturing, "llama2_decode_check: not allowed during graph capture");
+    int flag = 0;
+    L2_HIP(hipMemcpyAsync(&flag, d->state + kStateError, sizeof(int), hipMemcpyDeviceToHost, ctx().stream));
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    if (flag != 0)
+        return fail(LLAMA2_ERR_STEP_FAILED,
+                    "llama2_decode_check: a persistent step gave up waiting for data from another workgroup (its "
+                    "workgroups were not all resident, or the wait limit is too low); the decoder's results are "
+                    "undefined from that step on");
+    return LLAMA2_OK;
+}
+
+int llama2_decode_set_wait_limit(llama2_decoder* d, int polls)
+{
+    L2_REQUIRE_INIT();
+    L2_CHECK(d, "llama2_decode_set_wait_limit: null decoder");
+    L2_CHECK(polls >= 0, "llama2_decode_set_wait_limit: polls=%d must not be negative", polls);
+    L2_CHECK(!ctx().capturing, "llama2_decode_set_wait_limit: not allowed during graph capture");
+    if (d->persist_variant < 0)
+        return fail(LLAMA2_ERR_UNSUPPORTED, "llama2_decode_set_wait_limit: the decoder has no persistent step");
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    d->pa.spin_limit = polls;
+    for (auto& kind : d->graphs) { // the limit is a kernel argument of the captured persistent steps
+        if (kind[kPersistShape])
+            (void)hipGraphExecDestroy(kind[kPersistShape]);
+        kind[kPersistShape] = nullptr;
+    }
+    L2_HIP(hipMemsetAsync(d->state + kStateError, 0, sizeof(int), ctx().stream));
+    L2_HIP(hipStreamSynchronize(ctx().stream));
+    return LLAMA2_OK;
+}
+
+int llama2_decode_matvec_chain(llama2_decoder* d, const llama2_half* input, llama2_half* output)
+{
+    L2_REQUIRE_INIT();
+    const char* fn = "llama2_decode_matvec_chain";
+    L2_CHECK(d && input && output, "%s: null argument", fn);
+    L2_CHECK(aligned(input, 16) && aligned(output, 16), "%s: input and output must be 16-byte aligned", fn);
+    if (d->persist_variant < 0)
+        return fail(LLAMA2_ERR_UNSUPPORTED, "%s: the decoder was not created with LLAMA2_DECODE_PERSISTENT", fn);
+    hipLaunchKernelGGL(bump_serial_kernel, dim3(1), dim3(64), 0, ctx().stream, d->state);
+    L2_LAUNCH_CHECK("bump_serial_kernel");
+    PersistArgs a = d->pa;
+    a.skip_attention = 1;
+    a.embedding = nullptr, a.tokens = nullptr, a.x_in = input;
+    a.classifier = nullptr, a.logits = nullptr, a.x_out = output;
+    return persist_launch(d->persist_variant, a, ctx().num_cus);
 }
 
 int llama2_decode_destroy(llama2_decoder* d)

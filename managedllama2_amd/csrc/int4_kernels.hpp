@@ -171,6 +171,14 @@ __device__ __forceinline__ void rope_cos_sin(float& fcr, float& fci, int i, int 
     fci = sinf(val);
 }
 
+// The rotation of native/rope_kernel.cu:14-26 with the multiply-adds spelled out, so that every
+// kernel that inlines it rounds the same way.
+__device__ __forceinline__ void rope_rotate(float& o0, float& o1, float v0, float v1, float fcr, float fci)
+{
+    o0 = __builtin_fmaf(v0, fcr, -(v1 * fci));
+    o1 = __builtin_fmaf(v0, fci, v1 * fcr);
+}
+
 template <int J, int MODE, int STAGE>
 __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
 {
@@ -302,8 +310,7 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
                 float o0 = v0, o1 = v1;
                 if (t < 2) { // native/rope_kernel.cu:14-26
                     const float fcr = rope_tab[2 * i], fci = rope_tab[2 * i + 1];
-                    o0 = v0 * fcr - v1 * fci;
-                    o1 = v0 * fci + v1 * fcr;
+                    rope_rotate(o0, o1, v0, v1, fcr, fci);
                 }
                 dst[n0] = float_to_half_bits(o0);
                 dst[n0 + 64] = float_to_half_bits(o1);

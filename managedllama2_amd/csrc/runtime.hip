@@ -9,6 +9,8 @@
 namespace l2 {
 
 static Context g_ctx;
+// 32 heads x 64 blocks x (128 partial outputs + block max + block sum) floats
+constexpr size_t kAttnPartialsFloor = sizeof(float) * 32 * 64 * 130;
 static thread_local char g_err[512] = "";
 
 Context& ctx() { return g_ctx; }
@@ -36,15 +38,21 @@ int ensure_attn_partials(size_t bytes)
     if (c.capturing)
         return fail(LLAMA2_ERR_INVALID_ARGUMENT,
                     "scratch of %zu bytes must exist before graph capture starts (run the call once eagerly first)", bytes);
-    // Grow only between launches that use it: earlier kernels on the stream may
-    // still read the old buffer, so drain the stream first.
-    L2_HIP(hipStreamSynchronize(c.stream));
+    // The old buffer is never freed here: kernels already on the stream may still use it, and a
+    // graph the caller captured earlier keeps its address in its kernel arguments.  It is retired
+    // and released at llama2_shutdown.  Sizes at least double, so a handful of buffers covers any
+    // growth; the first request is rounded up to what a 32-head, 8192-row context needs.
+    size_t want = bytes < kAttnPartialsFloor ? kAttnPartialsFloor : bytes;
+    if (want < 2 * c.attn_partials_bytes)
+        want = 2 * c.attn_partials_bytes;
+    if (c.attn_partials && c.n_retired_partials >= kMaxRetiredPartials)
+        return fail(LLAMA2_ERR_UNSUPPORTED, "attention scratch grew more than %d times", kMaxRetiredPartials);
+    float* fresh = nullptr;
+    L2_HIP(hipMalloc(reinterpret_cast<void**>(&fresh), want));
     if (c.attn_partials)
-        L2_HIP(hipFree(c.attn_partials));
-    c.attn_partials = nullptr;
-    c.attn_partials_bytes = 0;
-    L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.attn_partials), bytes));
-    c.attn_partials_bytes = bytes;
+        c.retired_partials[c.n_retired_partials++] = c.attn_partials;
+    c.attn_partials = fresh;
+    c.attn_partials_bytes = want;
     return LLAMA2_OK;
 }
 
@@ -100,6 +108,10 @@ int llama2_init(int device)
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_keys), LLAMA2_MAX_SAMPLER_SIZE * sizeof(uint16_t)));
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_values), LLAMA2_MAX_SAMPLER_SIZE * sizeof(int)));
     c.device = device;
+    if (int rc = resolve_static_scratch(device)) {
+        c.device = -1;
+        return rc;
+    }
     c.ready = true;
     g_err[0] = 0;
     return LLAMA2_OK;
@@ -116,6 +128,9 @@ int llama2_shutdown(void)
         L2_HIP(hipFree(c.attn_partials));
     c.attn_partials = nullptr;
     c.attn_partials_bytes = 0;
+    for (int i = 0; i < c.n_retired_partials; ++i)
+        L2_HIP(hipFree(c.retired_partials[i]));
+    c.n_retired_partials = 0;
     if (c.attn_counters)
         L2_HIP(hipFree(c.attn_counters));
     c.attn_counters = nullptr;
