@@ -42,9 +42,6 @@ Context& ctx();
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char* what);
 int ensure_attn_partials(size_t bytes);
-// Resolves the device address of the file-scope scratch of llama2_multi_head_attention_static
-// (decode.hip) for `device`, which must be current; called once per device by llama2_init.
-int resolve_static_scratch(int device);
 // Sampler.Sample's stochastic branch in one launch (sampler.hip).  token_only: the caller reads the
 // token alone, so the sort may stop at the head of the distribution that holds top_p of the mass.
 int sample_launch(const char* fn, uint16_t* logits, int* indices, int size, float temperature, float top_p, float coin,
@@ -121,6 +118,21 @@ __device__ __forceinline__ float half_bits_to_float(uint16_t h)
 __device__ __forceinline__ uint16_t float_to_half_bits(float f)
 {
     return __builtin_bit_cast(uint16_t, static_cast<_Float16>(f)); // v_cvt_f16_f32, RNE
+}
+
+// The rotation of native/rope_kernel.cu:14-26, rounded the way the reference rounds it: the fp32
+// value first, then __float2half of it.  The multiply-adds are spelled out and the fp32 results are
+// made opaque before the conversion, so that every kernel that inlines this produces the same bits:
+// left alone, the compiler fuses some of these multiply-adds with the conversion (v_fma_mixlo_f16,
+// ONE rounding straight to fp16) and not others, depending on the surrounding code, and a value
+// near an fp16 tie then rounds differently from kernel to kernel.
+__device__ __forceinline__ void rope_rotate(uint16_t& b0, uint16_t& b1, float v0, float v1, float fcr, float fci)
+{
+    float o0 = __builtin_fmaf(v0, fcr, -(v1 * fci));
+    float o1 = __builtin_fmaf(v0, fci, v1 * fcr);
+    asm volatile("" : "+v"(o0), "+v"(o1));
+    b0 = float_to_half_bits(o0);
+    b1 = float_to_half_bits(o1);
 }
 
 // DPP controls (GCN3/CDNA encoding)

@@ -19,6 +19,7 @@
 #include "sampler_kernels.hpp"
 
 #include <climits>
+#include <cstdlib>
 #include <cmath>
 #include <new>
 #include <vector>
@@ -492,6 +493,11 @@ int persist_setup(llama2_decoder* d)
     a.state = d->state;
     a.spin_limit = kPersistSpinLimit;
     persist_bind_scratch(a, d->persist_scratch);
+#ifdef L2_PERSIST_TRACE
+    a.trace = nullptr;
+    if (const char* addr = getenv("LLAMA2_PERSIST_TRACE")) // a device buffer of n_layers * 4 * kPTracePoints 64-bit words
+        a.trace = reinterpret_cast<unsigned long long*>(strtoull(addr, nullptr, 0));
+#endif
     return LLAMA2_OK;
 }
 
@@ -716,7 +722,8 @@ int check_attention(const char* fn, const void* output, const void* query, const
 // blocks of a head and the heads' arrival counters live in this file-scope device
 // array (one copy per GPU, at its own address, for the life of the process).  In host
 // code the array's name is only a stand-in; its device address is asked for once per
-// device at llama2_init and every later use goes through that pointer.
+// device, at the entry point's first call there, and every later use goes through that
+// pointer.
 namespace l2 {
 struct StaticAttnScratch {
     float part[static_cast<size_t>(LLAMA2_STATIC_ATTENTION_BLOCKS) * kPartStride];
@@ -741,22 +748,32 @@ __global__ void clear_words_kernel(unsigned* p, int n)
         p[i] = 0u;
 }
 
-// Called by llama2_init with `device` current: resolves this device's copy of the array
-// and clears the arrival counters (the kernels leave them at zero after every launch).
+// Resolves the current device's copy of the array, once per device: asks the runtime for the
+// symbol's device address, makes sure that the runtime knows that address as device memory of this
+// device that covers the whole array (a wrong address must fail here, on the host, never in a
+// kernel), and clears the arrival counters (the kernels leave them at zero after every launch).
 int resolve_static_scratch(int device)
 {
     if (device < 0 || device >= kMaxDevices)
-        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_init: device %d beyond the %d the static scratch tracks", device,
-                    kMaxDevices);
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "device %d beyond the %d the static scratch tracks", device, kMaxDevices);
+    if (g_static_scratch[device])
+        return LLAMA2_OK;
     void* ptr = nullptr;
     L2_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-    if (!ptr)
-        return fail(LLAMA2_ERR_NO_DEVICE, "llama2_init: the static scratch has no address on device %d", device);
+    size_t bytes = 0;
+    L2_HIP(hipGetSymbolSize(&bytes, HIP_SYMBOL(scratch)));
+    if (!ptr || bytes != sizeof(StaticAttnScratch))
+        return fail(LLAMA2_ERR_NO_DEVICE, "the static scratch resolves to %p, %zu bytes on device %d (expected %zu bytes)",
+                    ptr, bytes, device, sizeof(StaticAttnScratch));
+    hipPointerAttribute_t attr{};
+    L2_HIP(hipPointerGetAttributes(&attr, ptr));
+    if (attr.type != hipMemoryTypeDevice || attr.device != device || attr.devicePointer != ptr)
+        return fail(LLAMA2_ERR_NO_DEVICE, "the static scratch address %p is not device memory of device %d (type %d, device %d)",
+                    ptr, device, static_cast<int>(attr.type), attr.device);
     StaticAttnScratch* sp = static_cast<StaticAttnScratch*>(ptr);
     hipLaunchKernelGGL(clear_words_kernel, dim3(ceil_div(kMaxAttnHeads, 256)), dim3(256), 0, ctx().stream, sp->counters,
                        kMaxAttnHeads);
     L2_LAUNCH_CHECK("clear_words_kernel");
-    L2_HIP(hipStreamSynchronize(ctx().stream));
     g_static_scratch[device] = sp;
     return LLAMA2_OK;
 }
@@ -792,9 +809,11 @@ int llama2_multi_head_attention_static(llama2_half* output, const llama2_half* q
     AttnShape shape{};
     L2_TRY(check_attention(fn, output, query, key, value, head_size, dim, seq_length, n_heads, &shape));
     StaticAttnScratch* sp = static_scratch_of(ctx().device);
-    if (!sp)
-        return fail(LLAMA2_ERR_NOT_INITIALIZED, "%s: the static scratch of device %d was not resolved at llama2_init", fn,
-                    ctx().device);
+    if (!sp) { // first call on this device
+        L2_CHECK(!ctx().capturing, "%s: call it once eagerly before capturing it into a graph", fn);
+        L2_TRY(resolve_static_scratch(ctx().device));
+        sp = static_scratch_of(ctx().device);
+    }
     if (static_cast<long long>(n_heads) * shape.splits > LLAMA2_STATIC_ATTENTION_BLOCKS)
         return fail(LLAMA2_ERR_UNSUPPORTED,
                     "%s: n_heads=%d x %d blocks of %d rows exceed the static scratch of %d (head, block) pairs; "

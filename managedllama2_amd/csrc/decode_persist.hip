@@ -33,6 +33,20 @@ constexpr int kPThreads = kPWaves * 64;
 __device__ __forceinline__ uint32_t tag16(uint32_t t) { return (t % 65535u) + 1u; } // never 0: a zeroed word is never ready
 __device__ __forceinline__ uint32_t tag32(uint32_t t) { return t | 0x80000000u; }
 
+// A pointer that is the same in every lane, moved to scalar registers.  The per-layer pointers
+// come from a table in device memory; the compiler cannot prove that nothing in this kernel writes
+// that table, loads it with vector loads, does the row arithmetic in vector registers -- and then
+// wraps every buffer load in a loop that makes its descriptor scalar again, a dozen instructions per
+// load.  One v_readfirstlane pair per descriptor avoids that.
+template <class T>
+__device__ __forceinline__ T* uniform_ptr(T* p)
+{
+    const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+    const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+    const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+    return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
+
 // One unsuccessful poll more.  Returns true when the wait has to be given up.
 __device__ __forceinline__ bool give_up(int* err, int& spins, int spin_limit)
 {
@@ -50,20 +64,21 @@ __device__ __forceinline__ bool give_up(int* err, int& spins, int spin_limit)
 }
 
 // Copies n tagged words (n % 4 == 0) from `src` into fp16 LDS vectors `dst` (and `dst2` if not
-// null) once each of them carries `tag`.  Threads [first, first + nthreads) of the workgroup
-// take part; each owns 16-byte pieces.
+// null) once each of them carries `tag`.  Called by the `nthreads` threads of a polling group
+// with their number t in it; each owns 16-byte pieces.
+// `src` is the same in every lane; `first_word` (a multiple of 4, may differ from lane to lane)
+// is where this thread's vector starts in it.
 __device__ __forceinline__ void poll_words(const uint32_t* src, int n, uint32_t tag, uint16_t* dst, uint16_t* dst2,
-                                           int first, int nthreads, int* err, int spin_limit)
+                                           int t, int nthreads, int* err, int spin_limit, int first_word = 0)
 {
-    const __amdgpu_buffer_rsrc_t r = make_rsrc(src, static_cast<uint32_t>(n) * 4u);
-    const int t = static_cast<int>(threadIdx.x) - first;
+    const __amdgpu_buffer_rsrc_t r = make_rsrc(uniform_ptr(src), 0x7FFFFFFCu);
     if (t < 0 || t >= nthreads)
         return;
     for (int p = t; p * 4 < n; p += nthreads) {
         u32x4 v;
         int spins = 0;
         for (;;) {
-            v = __builtin_amdgcn_raw_buffer_load_b128(r, p * 16, 0, kAuxAgent);
+            v = __builtin_amdgcn_raw_buffer_load_b128(r, (first_word + p * 4) * 4, 0, kAuxAgent);
             const uint32_t bad = ((v[0] >> 16) ^ tag) | ((v[1] >> 16) ^ tag) | ((v[2] >> 16) ^ tag) | ((v[3] >> 16) ^ tag);
             if (bad == 0u || give_up(err, spins, spin_limit))
                 break;
@@ -101,40 +116,88 @@ __device__ __forceinline__ float poll_part(const unsigned long long* src, uint32
     return __builtin_bit_cast(float, static_cast<uint32_t>(w));
 }
 
-// The first 256 threads turn the fp16 vector `raw` (LDS, K halfs) into the LDS image the int4
-// dot product reads (commit_pieces), optionally through RMSNorm with the preloaded weights
-// `gp`: the arithmetic of the 256-thread stand-alone kernels, order included.  All threads call.
+// commit_pieces of int4_kernels.hpp for thread `tid` of 256 (the caller's own copy of its thread
+// number, see the layer loop): the same LDS image, the same chunk sums.
 template <int J>
-__device__ __forceinline__ void stage_int4(const uint16_t* raw, int K, bool norm, const VecPieces<J>& gp, float eps,
-                                           u32x4* xs, float* sx, float* red4)
+__device__ __forceinline__ void commit_pieces_t(u32x4* xs, float* sx, const VecPieces<J>& p, int tid)
 {
-    const bool worker = threadIdx.x < 256;
-    VecPieces<J> xp;
+    constexpr int JC = J * 64;
 #pragma unroll
     for (int i = 0; i < J; ++i) {
-        const int e = threadIdx.x + i * 256;
+        const int e = tid + i * 256;
+        const u32x4 v = p.v[i];
+        u32x4 o;
+        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);     // x0,x4
+        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u); // x1,x5
+        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);     // x2,x6
+        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u); // x3,x7
+        xs[(e & 3) * JC + (e >> 2)] = o;
+        const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
+        s += dpp_f32<DPP_QUAD_XOR1>(s);
+        s += dpp_f32<DPP_QUAD_XOR2>(s);
+        if ((e & 3) == 0)
+            sx[e >> 2] = s;
+    }
+}
+
+// The first 256 threads turn the fp16 vector `raw` (LDS, K halfs) into the LDS image the int4
+// dot product reads, optionally through RMSNorm with the preloaded weights `gp`: the arithmetic
+// of the 256-thread stand-alone kernels, order included.  All threads call, with their number tid.
+template <int J>
+__device__ __forceinline__ void stage_int4(const uint16_t* raw, int K, bool norm, const uint16_t* gam, float eps,
+                                           u32x4* xs, float* sx, float* red4, int tid)
+{
+    const bool worker = tid < 256;
+    VecPieces<J> xp, gp;
+#pragma unroll
+    for (int i = 0; i < J; ++i) {
+        const int e = tid + i * 256;
         xp.v[i] = (worker && e * 8 < K) ? *reinterpret_cast<const u32x4*>(raw + e * 8) : u32x4{0u, 0u, 0u, 0u};
     }
     if (norm) { // uniform
         const float part = wave_sum(worker ? xp.sum_squares() : 0.0f);
-        if (worker && (threadIdx.x & 63) == 0)
-            red4[threadIdx.x >> 6] = part;
+        if (worker && (tid & 63) == 0)
+            red4[tid >> 6] = part;
         __syncthreads();
         const float ss = (red4[0] + red4[1]) + (red4[2] + red4[3]);
         const float rms = 1.0f / sqrtf(ss / static_cast<float>(K) + eps); // native/rmsnorm_kernel.cu:25-27
+#pragma unroll
+        for (int i = 0; i < J; ++i) {
+            const int e = tid + i * 256;
+            gp.v[i] = (worker && e * 8 < K) ? *reinterpret_cast<const u32x4*>(gam + e * 8) : u32x4{0u, 0u, 0u, 0u};
+        }
         xp.scale(rms, gp);
     }
     if (worker)
-        commit_pieces<J>(xs, sx, xp);
+        commit_pieces_t<J>(xs, sx, xp, tid);
     __syncthreads();
 }
 
+// RMSNorm weights on their way to LDS: requested by all threads before the wait for the input
+// vector (one 16-byte piece per thread and round), written to `gam` once that wait is over.
 template <int J>
-__device__ __forceinline__ void load_gamma(VecPieces<J>& gp, const uint16_t* gamma, int K)
-{
-    if (threadIdx.x < 256)
-        gp.load(gamma, K);
-}
+struct GammaPieces {
+    static constexpr int GP = (J * 256 + kPThreads - 1) / kPThreads;
+    u32x4 v[GP];
+    __device__ __forceinline__ void load(const uint16_t* gamma, int K, int tid)
+    {
+        const __amdgpu_buffer_rsrc_t r = make_rsrc(uniform_ptr(gamma), K * 2);
+#pragma unroll
+        for (int i = 0; i < GP; ++i)
+            v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, (tid + i * kPThreads) * 16, 0, 0);
+    }
+    __device__ __forceinline__ void store(uint16_t* gam, int tid) const
+    {
+#pragma unroll
+        for (int i = 0; i < GP; ++i)
+            if (tid + i * kPThreads < J * 256)
+                *reinterpret_cast<u32x4*>(gam + (tid + i * kPThreads) * 8) = v[i];
+    }
+};
 
 // What a lane keeps of R rows while they are in flight: J chunks of weights per row, and -- instead
 // of one zero word and one scale per chunk -- lane l's share of the row's zero words (word l) and
@@ -154,14 +217,14 @@ struct CFrag {
 // are unconditional on purpose: a conditional load makes the registers "old value or new value",
 // which keeps the previous round's registers alive across the whole layer.
 template <int J>
-__device__ __forceinline__ void load_row_c(u32x4 (&w)[J], uint32_t& zwv, uint32_t (&sbv)[(J + 3) / 4], const QW& m, int row,
+__device__ __forceinline__ void load_row_c(u32x4 (&w)[J], uint32_t& zwv, uint32_t (&sbv)[(J + 3) / 4], const QW m, int row,
                                            bool valid, int ws, int ss, int zs, int lane)
 {
     const size_t r = valid ? static_cast<size_t>(row) : 0;
     const uint32_t on = valid ? 1u : 0u;
-    const __amdgpu_buffer_rsrc_t rw = make_rsrc(m.w + r * ws, on * ws * 4);
-    const __amdgpu_buffer_rsrc_t rz = make_rsrc(m.z + r * zs, on * zs * 4);
-    const __amdgpu_buffer_rsrc_t rs = make_rsrc(m.s + r * ss, on * ss * 2);
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(uniform_ptr(m.w + r * ws), on * ws * 4);
+    const __amdgpu_buffer_rsrc_t rz = make_rsrc(uniform_ptr(m.z + r * zs), on * zs * 4);
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(uniform_ptr(m.s + r * ss), on * ss * 2);
 #pragma unroll
     for (int j = 0; j < J; ++j)
         w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
@@ -188,6 +251,14 @@ __device__ __forceinline__ void expand(Frag<J, R>& f, const CFrag<J, R>& c, int 
         }
 }
 
+// The per-layer pointer table is read through the constant address space: nothing writes it while
+// the kernel runs, and saying so lets the compiler fetch the pointers with scalar loads.  Read
+// through a plain pointer they would be vector loads -- and a vector load in the middle of the
+// weight stream makes the wavefront wait for every weight load it has in flight (loads complete in
+// order) before it can even form the next address.
+typedef const __attribute__((address_space(4))) PersistLayer* LayerTable;
+__device__ __forceinline__ QW table_qw(const __attribute__((address_space(4))) QW& q) { return QW{q.w, q.z, q.s}; }
+
 template <int JD, int JH, int RQ, int RO, int RS, int RD>
 __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a)
 {
@@ -201,6 +272,7 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
     // while a slow one still reads the previous
     __shared__ uint16_t xres[JD * 2048] __attribute__((aligned(16)));
     __shared__ uint16_t xres1[JD * 2048] __attribute__((aligned(16)));
+    __shared__ uint16_t gam[JD * 2048] __attribute__((aligned(16))); // RMSNorm weights of the stage at hand
     __shared__ float red4[4];
     __shared__ float rope_tab[kRopeHeadSize];
     __shared__ float sc[kPUnits][kPBlockRows];
@@ -210,10 +282,10 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
     __shared__ float mrg_w[64];
     __shared__ float mrg_l;
 
-    const int lane = threadIdx.x & 63;
+    const int lane0 = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
     const int G = gridDim.x, W = G * kPWaves;
-    const int gw = blockIdx.x * kPWaves + wave;
+    const int gw0 = blockIdx.x * kPWaves + wave;
     const int N = a.dim, NH = a.hidden, L = a.n_layers;
     const int nQ = 3 * N;
     const int wg0 = blockIdx.x * kPWaves; // the workgroup's first wavefront: it takes part in a phase iff wg0 < items
@@ -222,49 +294,68 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
     const int spin_limit = a.spin_limit;
     const int pos = a.state[kStatePos];
     const uint32_t tbase = static_cast<uint32_t>(a.state[kStateSerial]) * static_cast<uint32_t>(L + 2);
-    const int zshift = ((lane >> 2) & 7) * 4;
-
     if (threadIdx.x < kRopeHeadSize)
         rope_tab[threadIdx.x] = reinterpret_cast<const float*>(a.state + kStateInts)[threadIdx.x];
     __syncthreads();
+#ifdef L2_PERSIST_TRACE
+    const int trace_slot = blockIdx.x == 0 ? 0 : blockIdx.x == 1 ? 1 : blockIdx.x == 100 ? 2 : blockIdx.x == 255 ? 3 : -1;
+#define L2_TRACE(layer, point)                                                                                   \
+    do {                                                                                                         \
+        if (a.trace && trace_slot >= 0 && threadIdx.x == 0)                                                      \
+            a.trace[(static_cast<size_t>(layer) * 4 + trace_slot) * kPTracePoints + (point)] = __builtin_amdgcn_s_memrealtime(); \
+    } while (0)
+#else
+#define L2_TRACE(layer, point) do { } while (0)
+#endif
 
     // attention geometry of this step
     const int S = pos + 1; // attends rows 0..pos (src/Transformer.cs:175)
     const int nblk = (S + kPBlockRows - 1) / kPBlockRows;
     const int natt = a.skip_attention ? 0 : a.n_heads * nblk; // (head, block) items, taken kPUnits * G at a time
-    const int q4 = wave >> 2, wq = wave & 3, tq = threadIdx.x & 255; // q4: the attention unit of this wavefront
+    const int q4 = wave >> 2, wq = wave & 3; // q4: the attention unit of this wavefront
     const int mrg_h = G - 1 - static_cast<int>(blockIdx.x); // the head whose blocks this workgroup merges
     const bool wgM = !a.skip_attention && nblk > 1 && mrg_h < a.n_heads;
 
-    auto q_tensor = [&](const PersistLayer& P, int t) -> const QW& { return t == 0 ? P.q : (t == 1 ? P.k : P.v); };
-    auto issue_q_row = [&](CFrag<JD, 1> (&fq)[RQ], const PersistLayer& P, bool have_layer, int r) {
+    const LayerTable layers = (LayerTable)a.layers;
+    auto issue_q_row = [&](CFrag<JD, 1> (&fq)[RQ], int layer, bool have_layer, int r, int lane, int gw) {
         if (r < RQ) {
             const int it = gw + r * W;
             const int t = (it >= N) + (it >= 2 * N), n = it - t * N;
-            load_row_c<JD>(fq[r].w[0], fq[r].zwv[0], fq[r].sbv[0], q_tensor(P, t < 3 ? t : 2), n, have_layer && it < nQ, a.ws_d,
-                           a.ss_d, a.zs_d, lane);
+            const QW mq = table_qw(layers[layer].q), mk = table_qw(layers[layer].k), mv = table_qw(layers[layer].v);
+            const QW m = t == 0 ? mq : (t == 1 ? mk : mv);
+            load_row_c<JD>(fq[r].w[0], fq[r].zwv[0], fq[r].sbv[0], m, n, have_layer && it < nQ, a.ws_d, a.ss_d, a.zs_d, lane);
         }
     };
 
     CFrag<JD, 1> fq[RQ];
 #pragma unroll
     for (int r = 0; r < RQ; ++r)
-        issue_q_row(fq, a.layers[0], true, r);
+        issue_q_row(fq, 0, true, r, lane0, gw0);
 
     for (int l = 0; l < L; ++l) {
-        // an opaque copy of the lane number per layer: what is derived from it (the shuffle
-        // addresses of expand) is recomputed here instead of being kept in registers, or spilled,
-        // across the whole loop
-        int lane_l = lane;
-        asm volatile("" : "+v"(lane_l));
-        const PersistLayer& P = a.layers[l];
+        // Opaque copies of the thread and wavefront numbers, taken anew in every layer: whatever is
+        // derived from them (LDS and buffer addresses, shuffle indices, row numbers -- dozens of
+        // values) is recomputed per layer with a few scalar and vector instructions instead of being
+        // hoisted out of the loop, where it would occupy registers across the whole layer or be
+        // spilled to scratch memory -- and a reload from scratch waits behind every weight load the
+        // wavefront has in flight.
+        int tid_o = static_cast<int>(threadIdx.x), gw_o = gw0;
+        asm volatile("" : "+v"(tid_o));
+        asm volatile("" : "+s"(gw_o));
+        const int tid = tid_o, lane = tid & 63, tq = tid & 255, gw = gw_o;
+        const int zshift = ((lane >> 2) & 7) * 4;
+        const QW Po = table_qw(layers[l].o), Pgate = table_qw(layers[l].gate), Pup = table_qw(layers[l].up),
+                 Pdown = table_qw(layers[l].down);
+        const uint16_t* const rms_att = layers[l].rms_att;
+        const uint16_t* const rms_ffn = layers[l].rms_ffn;
         const uint32_t tag = tag16(tbase + static_cast<uint32_t>(l));
         const uint32_t tag_next = tag16(tbase + static_cast<uint32_t>(l) + 1u);
 
         // ------------------------------------------------ layer input: RMSNorm while staging
+        L2_TRACE(l, 0);
         if (wgQ) {
-            VecPieces<JD> gp;
-            load_gamma<JD>(gp, P.rms_att, N);
+            GammaPieces<JD> gp;
+            gp.load(rms_att, N, tid);
             if (l == 0) {
                 const uint16_t* src = a.x_in;
                 if (a.embedding) { // native/embedding_kernel.cu:9-11
@@ -272,50 +363,61 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
                     token = token < 0 ? 0 : (token >= a.vocab ? a.vocab - 1 : token); // never read outside the table
                     src = a.embedding + static_cast<size_t>(token) * N;
                 }
-                for (int p = threadIdx.x; p * 8 < N; p += kPThreads) {
+                for (int p = tid; p * 8 < N; p += kPThreads) {
                     const u32x4 v = *reinterpret_cast<const u32x4*>(src + p * 8);
                     *reinterpret_cast<u32x4*>(rawv + p * 8) = v;
                     *reinterpret_cast<u32x4*>(xres + p * 8) = v;
                 }
             } else {
-                poll_words(a.ll_x0, N, tag, rawv, xres, 0, kPThreads, err, spin_limit);
+                poll_words(a.ll_x0, N, tag, rawv, xres, tid, kPThreads, err, spin_limit);
             }
+            gp.store(gam, tid);
             __syncthreads();
-            stage_int4<JD>(rawv, N, true, gp, a.eps, xs, sx, red4);
+            L2_TRACE(l, 1);
+            stage_int4<JD>(rawv, N, true, gam, a.eps, xs, sx, red4, tid);
         }
+        L2_TRACE(l, 2);
 
         // o-proj rows and the first SwiGLU pair are requested now, two phases ahead of their use
         CFrag<JD, 1> fo[RO];
 #pragma unroll
         for (int r = 0; r < RO; ++r) {
             const int n = gw + r * W;
-            load_row_c<JD>(fo[r].w[0], fo[r].zwv[0], fo[r].sbv[0], P.o, n, n < N, a.ws_d, a.ss_d, a.zs_d, lane);
+            load_row_c<JD>(fo[r].w[0], fo[r].zwv[0], fo[r].sbv[0], Po, n, n < N, a.ws_d, a.ss_d, a.zs_d, lane);
         }
         CFrag<JD, 2> fs[RS];
         auto issue_s = [&](int r) {
             const int n = gw + r * W;
-            load_row_c<JD>(fs[r].w[0], fs[r].zwv[0], fs[r].sbv[0], P.gate, n, n < NH, a.ws_d, a.ss_d, a.zs_d, lane);
-            load_row_c<JD>(fs[r].w[1], fs[r].zwv[1], fs[r].sbv[1], P.up, n, n < NH, a.ws_d, a.ss_d, a.zs_d, lane);
+            load_row_c<JD>(fs[r].w[0], fs[r].zwv[0], fs[r].sbv[0], Pgate, n, n < NH, a.ws_d, a.ss_d, a.zs_d, lane);
+            load_row_c<JD>(fs[r].w[1], fs[r].zwv[1], fs[r].sbv[1], Pup, n, n < NH, a.ws_d, a.ss_d, a.zs_d, lane);
         };
         // SwiGLU pairs [0, S_A) are requested after the q/k/v rows are computed (in flight during
         // attention), [S_A, S_B) after the o-projection, the rest while earlier pairs are computed
-        constexpr int S_A = RS < 2 ? RS : 2, S_B = RS < 4 ? RS : 4;
+        constexpr int S_A = RS < 2 ? RS : 2, S_B = RS < 3 ? RS : 3;
 
         // ------------------------------------------------ q, k, v rows (unrotated, fp16) as tagged words
+        // The results of a phase are collected, row r in lane r, and stored once after the last row: a
+        // store issued between the rows would make every later wait for weights a wait for ALL memory
+        // operations in flight (loads and stores share one in-order counter and complete out of order
+        // with respect to each other), the freshly requested rows and the store's own
+        // acknowledgement included.  Nothing is lost: the consumers need the whole vector anyway.
+        uint32_t outw = 0;
 #pragma unroll
         for (int r = 0; r < RQ; ++r) {
             const int it = gw + r * W;
             if (it < nQ) {
                 float acc[1];
                 Frag<JD, 1> f;
-                expand<JD, 1>(f, fq[r], lane_l);
+                expand<JD, 1>(f, fq[r], lane);
                 dot_frag<JD, 1>(acc, f, xs, sx, lane, zshift);
                 const float v = wave_sum(acc[0]);
-                if (lane == 0)
-                    put_word(a.ll_qkv + it, tag, float_to_half_bits(v));
+                outw = lane == r ? float_to_half_bits(v) : outw;
             }
         }
+        if (lane < RQ && gw + lane * W < nQ)
+            put_word(a.ll_qkv + gw + lane * W, tag, static_cast<uint16_t>(outw));
 
+        L2_TRACE(l, 3);
 #pragma unroll
         for (int r = 0; r < S_A; ++r)
             issue_s(r);
@@ -345,18 +447,17 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
                 // this head's q, and for the last block the new k and v, 32 threads each
                 const int part = tq >> 5;
                 if (part < (last ? 3 : 1))
-                    poll_words(a.ll_qkv + part * N + att_h * kRopeHeadSize, kRopeHeadSize, tag, qkv_s[q4][part], nullptr,
-                               q4 * 256 + part * 32, 32, err, spin_limit);
+                    poll_words(a.ll_qkv, kRopeHeadSize, tag, qkv_s[q4][part], nullptr, tq - part * 32, 32, err, spin_limit,
+                               part * N + att_h * kRopeHeadSize);
             }
             __syncthreads();
             if (att_act) { // RoPE (native/rope_kernel.cu:3-26) and the cache row of this position
                 const int i = tq & 63, which = tq >> 6;
                 if (which == 0 || (which == 1 && last)) {
                     uint16_t* v = qkv_s[q4][which];
-                    float o0, o1;
-                    rope_rotate(o0, o1, half_bits_to_float(v[i]), half_bits_to_float(v[i + 64]), rope_tab[2 * i],
+                    uint16_t b0, b1;
+                    rope_rotate(b0, b1, half_bits_to_float(v[i]), half_bits_to_float(v[i + 64]), rope_tab[2 * i],
                                 rope_tab[2 * i + 1]);
-                    const uint16_t b0 = float_to_half_bits(o0), b1 = float_to_half_bits(o1);
                     v[i] = b0;
                     v[i + 64] = b1;
                     if (which == 1) {
@@ -482,52 +583,58 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
         }
 
         // ------------------------------------------------ o-proj + residual
+        L2_TRACE(l, 4);
         if (wgO) {
-            const VecPieces<JD> none{};
-            poll_words(a.skip_attention ? a.ll_qkv : a.ll_att, N, tag, rawv, nullptr, 0, kPThreads, err, spin_limit);
+            poll_words(a.skip_attention ? a.ll_qkv : a.ll_att, N, tag, rawv, nullptr, tid, kPThreads, err, spin_limit);
             __syncthreads();
-            stage_int4<JD>(rawv, N, false, none, a.eps, xs, sx, red4);
+            L2_TRACE(l, 5);
+            stage_int4<JD>(rawv, N, false, gam, a.eps, xs, sx, red4, tid);
         }
+        L2_TRACE(l, 6);
 #pragma unroll
         for (int r = 0; r < RO; ++r) {
             const int n = gw + r * W;
             if (n < N) {
                 float acc[1];
                 Frag<JD, 1> f;
-                expand<JD, 1>(f, fo[r], lane_l);
+                expand<JD, 1>(f, fo[r], lane);
                 dot_frag<JD, 1>(acc, f, xs, sx, lane, zshift);
                 float v = wave_sum(acc[0]);
-                if (lane == 0) {
-                    v += half_bits_to_float(xres[n]);
-                    put_word(a.ll_x1 + n, tag, float_to_half_bits(v));
-                }
+                v += half_bits_to_float(xres[n]);
+                outw = lane == r ? float_to_half_bits(v) : outw;
             }
         }
+        if (lane < RO && gw + lane * W < N)
+            put_word(a.ll_x1 + gw + lane * W, tag, static_cast<uint16_t>(outw));
 #pragma unroll
         for (int r = S_A; r < S_B; ++r)
             issue_s(r);
 
         // ------------------------------------------------ RMSNorm + SwiGLU
+        L2_TRACE(l, 7);
         if (wgS) { // every workgroup with down-proj rows has SwiGLU rows too (hidden >= dim: checked on the host)
-            VecPieces<JD> gp;
-            load_gamma<JD>(gp, P.rms_ffn, N);
-            poll_words(a.ll_x1, N, tag, rawv, xres1, 0, kPThreads, err, spin_limit);
+            GammaPieces<JD> gp;
+            gp.load(rms_ffn, N, tid);
+            poll_words(a.ll_x1, N, tag, rawv, xres1, tid, kPThreads, err, spin_limit);
+            gp.store(gam, tid);
             __syncthreads();
-            stage_int4<JD>(rawv, N, true, gp, a.eps, xs, sx, red4);
+            L2_TRACE(l, 8);
+            stage_int4<JD>(rawv, N, true, gam, a.eps, xs, sx, red4, tid);
         }
+        L2_TRACE(l, 9);
         CFrag<JH, 1> fd[RD];
         constexpr int NS2 = RS - S_B, NI = NS2 + RD + RQ, PER = (NI + RS - 1) / RS;
         const bool have_next = l + 1 < L;
-        const PersistLayer& PN = a.layers[have_next ? l + 1 : l];
+        const int next_layer = have_next ? l + 1 : l;
         auto issue_ahead = [&](int i) {
             if (i < NS2) {
                 issue_s(S_B + i);
             } else if (i < NS2 + RD) {
                 const int nd = gw + (i - NS2) * W;
-                load_row_c<JH>(fd[i - NS2].w[0], fd[i - NS2].zwv[0], fd[i - NS2].sbv[0], P.down, nd, nd < N, a.ws_h, a.ss_h,
+                load_row_c<JH>(fd[i - NS2].w[0], fd[i - NS2].zwv[0], fd[i - NS2].sbv[0], Pdown, nd, nd < N, a.ws_h, a.ss_h,
                                a.zs_h, lane);
             } else if (i < NI) {
-                issue_q_row(fq, PN, have_next, i - NS2 - RD);
+                issue_q_row(fq, next_layer, have_next, i - NS2 - RD, lane, gw);
             }
         };
 #pragma unroll
@@ -536,15 +643,13 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
             if (n < NH) {
                 float acc[2];
                 Frag<JD, 2> f;
-                expand<JD, 2>(f, fs[r], lane_l);
+                expand<JD, 2>(f, fs[r], lane);
                 dot_frag<JD, 2>(acc, f, xs, sx, lane, zshift);
                 const float g = wave_sum(acc[0]), u = wave_sum(acc[1]);
-                if (lane == 0) {
-                    float v = g;
-                    v *= 1.0f / (1.0f + expf(-v)); // native/mat_vec_kernel.cu:219-221
-                    v *= u;
-                    put_word(a.ll_h + n, tag, float_to_half_bits(v));
-                }
+                float v = g;
+                v *= 1.0f / (1.0f + expf(-v)); // native/mat_vec_kernel.cu:219-221
+                v *= u;
+                outw = lane == r ? float_to_half_bits(v) : outw;
             }
             // the registers a computed pair frees take, in this order, the remaining pairs, the down-proj
             // rows and the next layer's q/k/v rows, PER of them per pair
@@ -555,36 +660,42 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
 #pragma unroll
         for (int i = RS * PER; i < NI; ++i)
             issue_ahead(i);
+        if (lane < RS && gw + lane * W < NH)
+            put_word(a.ll_h + gw + lane * W, tag, static_cast<uint16_t>(outw));
 
         // ------------------------------------------------ down-proj + residual
+        L2_TRACE(l, 10);
         if (wgO) {
-            const VecPieces<JH> none{};
-            poll_words(a.ll_h, NH, tag, rawv, nullptr, 0, kPThreads, err, spin_limit);
+            poll_words(a.ll_h, NH, tag, rawv, nullptr, tid, kPThreads, err, spin_limit);
             __syncthreads();
-            stage_int4<JH>(rawv, NH, false, none, a.eps, xs, sx, red4);
+            L2_TRACE(l, 11);
+            stage_int4<JH>(rawv, NH, false, gam, a.eps, xs, sx, red4, tid);
         }
+        L2_TRACE(l, 12);
 #pragma unroll
         for (int r = 0; r < RD; ++r) {
             const int n = gw + r * W;
             if (n < N) {
                 float acc[1];
                 Frag<JH, 1> f;
-                expand<JH, 1>(f, fd[r], lane_l);
+                expand<JH, 1>(f, fd[r], lane);
                 dot_frag<JH, 1>(acc, f, xs, sx, lane, zshift);
                 float v = wave_sum(acc[0]);
-                if (lane == 0) {
-                    v += half_bits_to_float(xres1[n]);
-                    put_word(a.ll_x0 + n, tag_next, float_to_half_bits(v));
-                }
+                v += half_bits_to_float(xres1[n]);
+                outw = lane == r ? float_to_half_bits(v) : outw;
             }
         }
+        if (lane < RD && gw + lane * W < N)
+            put_word(a.ll_x0 + gw + lane * W, tag_next, static_cast<uint16_t>(outw));
+        L2_TRACE(l, 13);
     }
 
     // ---------------------------------------------------- final RMSNorm + classifier (src/Transformer.cs:187-189)
+    const int lane = lane0, gw = gw0;
     const uint32_t tag = tag16(tbase + static_cast<uint32_t>(L));
     if (!a.classifier) {
         if (blockIdx.x == 0) { // the mat-vec chain alone: hand the residual stream back as plain fp16
-            poll_words(a.ll_x0, N, tag, rawv, nullptr, 0, kPThreads, err, spin_limit);
+            poll_words(a.ll_x0, N, tag, rawv, nullptr, static_cast<int>(threadIdx.x), kPThreads, err, spin_limit);
             __syncthreads();
             for (int p = threadIdx.x; p * 8 < N; p += kPThreads)
                 *reinterpret_cast<u32x4*>(a.x_out + p * 8) = *reinterpret_cast<const u32x4*>(rawv + p * 8);
@@ -596,7 +707,8 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
     const int nchunks = N >> 3;
     u32x4 cur[CL], nxt[CL];
     auto issue_row = [&](u32x4 (&m)[CL], int n) {
-        const __amdgpu_buffer_rsrc_t rm = make_rsrc(a.classifier + static_cast<size_t>(n) * N, static_cast<uint32_t>(N) * 2u);
+        const __amdgpu_buffer_rsrc_t rm =
+            make_rsrc(uniform_ptr(a.classifier + static_cast<size_t>(n) * N), static_cast<uint32_t>(N) * 2u);
 #pragma unroll
         for (int u = 0; u < CL; ++u)
             m[u] = __builtin_amdgcn_raw_buffer_load_b128(rm, (lane + 64 * u) * 16, 0, kAuxNonTemporal);
@@ -605,8 +717,10 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
         issue_row(cur, gw);
     {
         VecPieces<JD> gp, xp;
-        load_gamma<JD>(gp, a.rms_final, N);
-        poll_words(a.ll_x0, N, tag, rawv, nullptr, 0, kPThreads, err, spin_limit);
+        GammaPieces<JD> gq;
+        gq.load(a.rms_final, N, static_cast<int>(threadIdx.x));
+        poll_words(a.ll_x0, N, tag, rawv, nullptr, static_cast<int>(threadIdx.x), kPThreads, err, spin_limit);
+        gq.store(gam, static_cast<int>(threadIdx.x));
         __syncthreads();
         const bool worker = threadIdx.x < 256;
 #pragma unroll
@@ -620,6 +734,11 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
         __syncthreads();
         const float ss = (red4[0] + red4[1]) + (red4[2] + red4[3]);
         const float rms = 1.0f / sqrtf(ss / static_cast<float>(N) + a.eps);
+#pragma unroll
+        for (int i = 0; i < JD; ++i) {
+            const int e = threadIdx.x + i * 256;
+            gp.v[i] = (worker && e * 8 < N) ? *reinterpret_cast<const u32x4*>(gam + e * 8) : u32x4{0u, 0u, 0u, 0u};
+        }
         xp.scale(rms, gp);
         if (worker) {
 #pragma unroll
@@ -631,7 +750,9 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
         }
         __syncthreads();
     }
-    for (int n = gw; n < a.vocab; n += W) {
+    uint32_t outw = 0; // logits of this wavefront's rows, row k in lane k % 64, stored 64 at a time
+    int k = 0;
+    for (int n = gw; n < a.vocab; n += W, ++k) {
         const int nn = n + W;
         if (nn < a.vocab)
             issue_row(nxt, nn);
@@ -647,8 +768,12 @@ __global__ __launch_bounds__(kPThreads) void decode_persist_kernel(PersistArgs a
             }
         }
         const float sum = wave_sum(acc);
-        if (lane == 0)
-            a.logits[n] = float_to_half_bits(sum);
+        outw = lane == (k & 63) ? float_to_half_bits(sum) : outw;
+        if ((k & 63) == 63 || nn >= a.vocab) {
+            const int row = gw + ((k & ~63) + lane) * W;
+            if (lane <= (k & 63))
+                a.logits[row] = static_cast<uint16_t>(outw);
+        }
 #pragma unroll
         for (int u = 0; u < CL; ++u)
             cur[u] = nxt[u];

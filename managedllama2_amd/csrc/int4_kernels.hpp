@@ -171,14 +171,6 @@ __device__ __forceinline__ void rope_cos_sin(float& fcr, float& fci, int i, int 
     fci = sinf(val);
 }
 
-// The rotation of native/rope_kernel.cu:14-26 with the multiply-adds spelled out, so that every
-// kernel that inlines it rounds the same way.
-__device__ __forceinline__ void rope_rotate(float& o0, float& o1, float v0, float v1, float fcr, float fci)
-{
-    o0 = __builtin_fmaf(v0, fcr, -(v1 * fci));
-    o1 = __builtin_fmaf(v0, fci, v1 * fcr);
-}
-
 template <int J, int MODE, int STAGE>
 __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
 {
@@ -307,13 +299,11 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
                 const int t = (item >= pairs) + (item >= 2 * pairs), rem = item - t * pairs;
                 const int i = rem & 63, n0 = (rem >> 6) * kRopeHeadSize + i;
                 uint16_t* dst = t == 0 ? a.out[0] : a.out[t] + static_cast<size_t>(pos) * a.kv_dim;
-                float o0 = v0, o1 = v1;
-                if (t < 2) { // native/rope_kernel.cu:14-26
-                    const float fcr = rope_tab[2 * i], fci = rope_tab[2 * i + 1];
-                    rope_rotate(o0, o1, v0, v1, fcr, fci);
-                }
-                dst[n0] = float_to_half_bits(o0);
-                dst[n0 + 64] = float_to_half_bits(o1);
+                uint16_t b0 = float_to_half_bits(v0), b1 = float_to_half_bits(v1);
+                if (t < 2) // native/rope_kernel.cu:14-26
+                    rope_rotate(b0, b1, v0, v1, rope_tab[2 * i], rope_tab[2 * i + 1]);
+                dst[n0] = b0;
+                dst[n0 + 64] = b1;
             }
         } else {
             float v = wave_sum(acc[0]);

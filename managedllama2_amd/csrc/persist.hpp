@@ -57,7 +57,13 @@ struct PersistArgs {
     unsigned long long* ll_part; // [n_heads][kPMaxBlocks][kPPartStride] attention partials
     int skip_attention; // 1: the o-projection consumes q directly (mat-vec chain without attention)
     int spin_limit;     // polls before a wait gives up and raises the error flag
+#ifdef L2_PERSIST_TRACE
+    // diagnostic build (make TRACE=1): wavefront 0 of workgroups 0, 1, 100 and 255 stores the
+    // 100 MHz clock at every phase boundary, kPTracePoints records per layer and workgroup
+    unsigned long long* trace;
+#endif
 };
+constexpr int kPTracePoints = 16;
 
 // Index of the kernel instantiation that fits the shapes on `num_cus` compute units, or -1.
 int persist_variant(int dim, int hidden, int n_heads, int num_cus);

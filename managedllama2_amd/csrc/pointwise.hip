@@ -88,14 +88,9 @@ __global__ void rope_kernel(uint16_t* q, uint16_t* k, int n_kv_heads, int head_s
         const float val = static_cast<float>(pos) * freq;
         const float fcr = cosf(val);
         const float fci = sinf(val);
-        const float q0 = half_bits_to_float(q[i]), q1 = half_bits_to_float(q[j]);
-        q[i] = float_to_half_bits(q0 * fcr - q1 * fci);
-        q[j] = float_to_half_bits(q0 * fci + q1 * fcr);
-        if (static_cast<int>(blockIdx.x) < n_kv_heads) {
-            const float k0 = half_bits_to_float(k[i]), k1 = half_bits_to_float(k[j]);
-            k[i] = float_to_half_bits(k0 * fcr - k1 * fci);
-            k[j] = float_to_half_bits(k0 * fci + k1 * fcr);
-        }
+        rope_rotate(q[i], q[j], half_bits_to_float(q[i]), half_bits_to_float(q[j]), fcr, fci);
+        if (static_cast<int>(blockIdx.x) < n_kv_heads)
+            rope_rotate(k[i], k[j], half_bits_to_float(k[i]), half_bits_to_float(k[j]), fcr, fci);
     }
 }
 

@@ -108,10 +108,6 @@ int llama2_init(int device)
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_keys), LLAMA2_MAX_SAMPLER_SIZE * sizeof(uint16_t)));
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_values), LLAMA2_MAX_SAMPLER_SIZE * sizeof(int)));
     c.device = device;
-    if (int rc = resolve_static_scratch(device)) {
-        c.device = -1;
-        return rc;
-    }
     c.ready = true;
     g_err[0] = 0;
     return LLAMA2_OK;
