@@ -11,9 +11,14 @@ hipGraph so the host's per-call cost never bounds what the GPU does.
 
 Prints ONE JSON line: whole-job HBM GB/s over the algorithmic bytes of the
 mat-vec set (`value`), the roofline record of the dominant kernel (fused
-SwiGLU), decode attention GB/s at 512/2048/4096 rows, full greedy decode
+SwiGLU), the single 4096x4096 mat-vec (configs[0]) and the 13B layer set
+(configs[2]), decode attention GB/s at 512/2048/4096 rows, full greedy decode
 tokens/s (128-token prompt + 256 generated tokens), and the reference's
 single-threaded C# CPU path (restated in C) timed beside it.
+
+Every timed figure comes from at least 100 graph replays after warm-up (HIP
+events on the library's stream), with the spread (p10 / median / p90) over at
+least 50 replays timed one by one; `steps` is what was really timed.
 """
 import argparse
 import ctypes as C
@@ -30,8 +35,13 @@ sys.path.insert(0, ROOT)
 
 # HBM bytes per launch of the dominant kernel (fused SwiGLU, 46 880 256 algorithmic bytes), measured with
 # two rocprofv3 --pmc runs of `bench.py --only kernel,calib` (counters cannot be read from inside this
-# process): (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000) x 1024
+# process): (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000) x 1024.  The figure belongs to one state of the
+# kernel's source: when csrc/int4_kernels.hpp no longer hashes to the value below, the kernel has changed
+# since the counters were read and `roofline.traffic` is reported as null until they are read again.
 SWIGLU_HBM_TRAFFIC_BYTES = 47409114
+SWIGLU_HBM_TRAFFIC_SOURCE_SHA16 = "@@SHA16@@"
+MIN_REPLAYS = 100   # graph replays behind every headline figure
+MIN_SAMPLES = 50    # replays timed one by one for the spread
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
 
 
@@ -62,14 +72,17 @@ def main():
     ap.add_argument("--steps", type=int, default=3200)
     ap.add_argument("--warmup", type=int, default=320)
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
-    ap.add_argument("--only", default="", help="comma list of legs: set,kernel,calib,attn,decode,sampler,repack,cpu (default: all but calib)")
-    ap.add_argument("--decode-mode", default="fused_graph", choices=["modules", "fused", "fused_graph"])
+    ap.add_argument("--only", default="", help="comma list of legs: set,kernel,cfg0,cfg2,calib,attn,chain,decode,sampler,repack,cpu "
+                                               "(default: all but calib)")
+    ap.add_argument("--decode-mode", default="fused_graph",
+                    choices=["modules", "fused", "fused_graph", "persistent", "persistent_graph"])
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (batch-1 decode has no cross-GPU exchange to measure); "
             "--gpus %d is not supported" % args.gpus)
         sys.exit(2)
-    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "attn", "decode", "sampler", "repack", "cpu"}
+    legs = set(args.only.split(",")) if args.only else {"set", "kernel", "cfg0", "cfg2", "attn", "chain", "decode", "sampler",
+                                                        "repack", "cpu"}
 
     from managedllama2_amd import capi, synth
     from managedllama2_amd.device import DeviceVariable, init
@@ -98,7 +111,9 @@ def main():
             "classifier": synth.normal_f16(rng, cfg["vocab_size"] * dim, 0.02),
             "rms_final": np.ones(dim, np.float16), "layers": lazy_layers()}
     mode = {"modules": capi.DECODE_MODULES, "fused": capi.DECODE_FUSED,
-            "fused_graph": capi.DECODE_FUSED | capi.DECODE_GRAPH}[args.decode_mode]
+            "fused_graph": capi.DECODE_FUSED | capi.DECODE_GRAPH,
+            "persistent": capi.DECODE_FUSED | capi.DECODE_PERSISTENT,
+            "persistent_graph": capi.DECODE_FUSED | capi.DECODE_PERSISTENT | capi.DECODE_GRAPH}[args.decode_mode]
     model = Transformer(cfg, host, mode=mode)
     del host
     layers = model.weights.layers
@@ -162,6 +177,21 @@ def main():
         capi.call("llama2_sync")
         return ms
 
+    def measure(graph, units_per_replay, replays=MIN_REPLAYS, warmup=3):
+        """Mean microseconds per unit over `replays` (>= MIN_REPLAYS) back-to-back replays, and the
+        p10 / median / p90 over MIN_SAMPLES replays timed one by one."""
+        replays = max(replays, MIN_REPLAYS)
+        for _ in range(max(warmup, 1)):
+            capi.call("llama2_graph_launch", graph)
+        us = 1e3 * timed_replays(graph, replays) / (replays * units_per_replay)
+        one_by_one = []
+        for _ in range(MIN_SAMPLES):
+            ev.start()
+            capi.call("llama2_graph_launch", graph)
+            one_by_one.append(1e3 * ev.stop_ms() / units_per_replay)
+        spread = [round(float(v), 3) for v in np.percentile(np.array(one_by_one), [10, 50, 90])]
+        return us, spread, replays
+
     result = {
         "metric": "int4 mat-vec HBM GB/s, Llama-2-7B decoder-layer mat-vec set, batch 1",
         "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -173,53 +203,128 @@ def main():
     }
 
     if "set" in legs:
-        # one graph = one pass over all distinct layers; K steps = K / n_layers replays
+        # one graph = one pass over all distinct layers; K steps = K / n_layers replays, at least MIN_REPLAYS
         graph = capture(step, n_layers)
-        replays = max(args.steps // n_layers, 1)
-        steps = replays * n_layers
-        for _ in range(max(args.warmup // n_layers, 1)):
-            capi.call("llama2_graph_launch", graph)
-        capi.call("llama2_sync")
         wall0 = time.perf_counter()
-        ms = timed_replays(graph, replays)
+        us, spread, replays = measure(graph, n_layers, replays=-(-args.steps // n_layers),
+                                      warmup=max(args.warmup // n_layers, 1))
         wall = time.perf_counter() - wall0
-        # the spread over replays (one replay = one pass over the 32 layers), each timed on its own
-        per_replay = []
-        for _ in range(min(replays, 50)):
-            ev.start()
-            capi.call("llama2_graph_launch", graph)
-            per_replay.append(ev.stop_ms() / n_layers)
-        spread = np.percentile(np.array(per_replay), [10, 50, 90])
         capi.call("llama2_graph_destroy", graph)
-        ms_per_step = ms / steps
+        steps = replays * n_layers
+        ms_per_step = us * 1e-3
         gbps = sizes["total"] / (ms_per_step * 1e-3) / 1e9
-        result.update(steps=steps, value=round(gbps, 1), ms_per_step=round(ms_per_step, 5),
-                      pct_of_hbm_peak=round(100 * gbps / HBM_PEAK_GBPS, 2),
-                      wall_ms_per_step=round(1e3 * wall / steps, 5),
-                      ms_per_step_p10_median_p90=[round(float(v), 5) for v in spread])
-        log("layer mat-vec set: %.2f us/step, %.0f GB/s (%.1f%% of 8 TB/s)" %
-            (1e3 * ms_per_step, gbps, 100 * gbps / HBM_PEAK_GBPS))
+        result.update(steps=steps, steps_requested=args.steps, replays=replays, value=round(gbps, 1),
+                      ms_per_step=round(ms_per_step, 5), pct_of_hbm_peak=round(100 * gbps / HBM_PEAK_GBPS, 2),
+                      wall_ms_per_step_incl_spread_runs=round(1e3 * wall / (steps + MIN_SAMPLES * n_layers), 5),
+                      us_per_step_p10_median_p90=spread, spread_samples=MIN_SAMPLES)
+        log("layer mat-vec set: %.2f us/step over %d replays (p10 %.2f / median %.2f / p90 %.2f), %.0f GB/s (%.1f%% of 8 TB/s)" %
+            (us, replays, spread[0], spread[1], spread[2], gbps, 100 * gbps / HBM_PEAK_GBPS))
 
     if "kernel" in legs:
         per_kernel = {}
         for name, fn in (("qkv", qkv), ("o", oproj), ("swiglu", swiglu), ("down", down)):
             graph = capture(lambda i, fn=fn: fn(layers[i % n_layers]), n_layers)
-            replays = max(args.steps // n_layers // 2, 2)
-            capi.call("llama2_graph_launch", graph)
-            us = 1e3 * timed_replays(graph, replays) / (replays * n_layers)
+            us, spread, replays = measure(graph, n_layers)
             capi.call("llama2_graph_destroy", graph)
-            per_kernel[name] = {"us": round(us, 3), "GBps": round(sizes[name] / us / 1e3, 1),
-                                "bytes": sizes[name]}
+            per_kernel[name] = {"us": round(us, 3), "us_p10_median_p90": spread, "launches": replays * n_layers,
+                                "GBps": round(sizes[name] / us / 1e3, 1), "bytes": sizes[name],
+                                "frac_of_hbm_peak": round(sizes[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
             log("  %-7s %8.2f us  %7.0f GB/s  (%d B)" % (name, us, sizes[name] / us / 1e3, sizes[name]))
         dom = per_kernel["swiglu"]
+        import hashlib
+        src = os.path.join(ROOT, "managedllama2_amd", "csrc", "int4_kernels.hpp")
+        sha16 = hashlib.sha256(open(src, "rb").read()).hexdigest()[:16] if os.path.exists(src) else None
+        fresh = sha16 == SWIGLU_HBM_TRAFFIC_SOURCE_SHA16
         result["roofline"] = {"bound": "hbm", "kernel": "int4_matvec_kernel<2, SWIGLU> (fused gate/up, 2x11008x4096)",
                               "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                              "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4), "traffic": SWIGLU_HBM_TRAFFIC_BYTES,
-                              "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, scaled by a "
-                                                "1 GiB copy kernel (factors 2.000 / 1.000): profiles/"
-                                                "int4_matvec_7b_layer_set_hbm_traffic.md",
-                              "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_us": dom["us"]}
+                              "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
+                              "traffic": SWIGLU_HBM_TRAFFIC_BYTES if fresh else None,
+                              "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of `bench.py --only kernel,calib`, "
+                                                "scaled by a 1 GiB copy kernel (factors 2.000 / 1.000): profiles/"
+                                                "int4_matvec_7b_layer_set_hbm_traffic.md; read for the kernel source "
+                                                "with sha256[:16] = %s, this run's source: %s%s" %
+                                                (SWIGLU_HBM_TRAFFIC_SOURCE_SHA16, sha16,
+                                                 "" if fresh else " (changed since: counters not re-read, traffic withheld)"),
+                              "algorithmic_bytes_per_launch": dom["bytes"], "avg_launch_us": dom["us"],
+                              "launches_timed": dom["launches"]}
         result["per_kernel"] = per_kernel
+
+    if "cfg0" in legs:
+        # configs[0]: ONE int4 mat-vec 4096 x 4096 (plain, and with the residual epilogue), cycled over the
+        # model's 128 distinct q / k / v / o tensors (1.1 GB: cold HBM).  8 732 672 algorithmic bytes
+        # (+ 8 192 for the residual read); floor at 8 TB/s: 1.09 us.
+        tensors = [w for L in layers for w in (L.queryWeight, L.keyWeight, L.valueWeight, L.outputWeight)]
+        b0 = synth.qweight_bytes(dim, dim) + 2 * dim + 2 * dim
+        cfg0 = {}
+        for name, entry, nbytes in (("plain", "llama2_mat_vec_int4", b0), ("residual", "llama2_mat_vec_residual_int4", b0 + 2 * dim)):
+            graph = capture(lambda i, entry=entry: capi.call(entry, x.ptr, xb.ptr, tensors[i].Weight.ptr, tensors[i].Zeros.ptr,
+                                                              tensors[i].Scales.ptr, dim, dim, zs, ss, ws), len(tensors))
+            us, spread, replays = measure(graph, len(tensors))
+            capi.call("llama2_graph_destroy", graph)
+            cfg0[name] = {"us": round(us, 3), "us_p10_median_p90": spread, "launches": replays * len(tensors), "bytes": nbytes,
+                          "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
+                          "floor_us_at_8TBps": round(nbytes / 8e6, 3)}
+            log("  cfg0 %-9s %6.2f us  %6.0f GB/s (%.1f%% of peak; floor %.2f us)" %
+                (name, us, nbytes / us / 1e3, 100 * nbytes / us / 1e3 / HBM_PEAK_GBPS, nbytes / 8e6))
+        cfg0["workload"] = "configs[0]: single AWQ int4 mat-vec K = N = 4096, %d distinct tensors cycled" % len(tensors)
+        result["cfg0"] = cfg0
+
+    if "cfg2" in legs:
+        # configs[2]: the Llama-2-13B layer mat-vec set (dim 5120, hidden 13824; 14 padded zero words per
+        # down-proj row) over 4 distinct layers (660 MB: cold HBM).  164 960 256 algorithmic bytes; floor 20.6 us.
+        d13, h13, n13 = synth.LLAMA2_13B["dim"], synth.LLAMA2_13B["hidden_dim"], 4
+        s13 = synth.layer_matvec_set_bytes(d13, h13)
+        z13, q13, w13 = (lambda t: (t[2], t[1], t[0]))(synth.qweight_sizes(d13))
+        hz13, hq13, hw13 = (lambda t: (t[2], t[1], t[0]))(synth.qweight_sizes(h13))
+        from managedllama2_amd.device import QWeight
+        rng13 = synth.rng_for(2, 13)
+        L13 = []
+        for _ in range(n13):
+            hl = synth.random_layer(rng13, d13, h13)
+            L13.append({k: QWeight.from_host(*hl[k]) for k in ("q", "k", "v", "o", "gate", "up", "down")})
+        xb13 = DeviceVariable.from_host(synth.normal_f16(rng13, d13))
+        x13, q13v, k13v, v13v = (DeviceVariable.zeros(np.float16, d13) for _ in range(4))
+        hbuf13 = DeviceVariable.zeros(np.float16, h13)
+
+        def p3(w):
+            return (w.Weight.ptr, w.Zeros.ptr, w.Scales.ptr)
+
+        def qkv13(L):
+            capi.call("llama2_qkv_mat_vec", q13v.ptr, k13v.ptr, v13v.ptr, xb13.ptr, *p3(L["q"]), *p3(L["k"]), *p3(L["v"]),
+                      d13, d13, z13, q13, w13)
+
+        def o13(L):
+            capi.call("llama2_mat_vec_residual_int4", x13.ptr, xb13.ptr, *p3(L["o"]), d13, d13, z13, q13, w13)
+
+        def sw13(L):
+            capi.call("llama2_mat_vec_swiglu", hbuf13.ptr, xb13.ptr, *p3(L["gate"]), *p3(L["up"]), d13, h13, z13, q13, w13)
+
+        def dn13(L):
+            capi.call("llama2_mat_vec_residual_int4", x13.ptr, hbuf13.ptr, *p3(L["down"]), h13, d13, hz13, hq13, hw13)
+
+        cfg2 = {"workload": "configs[2]: 13B layer mat-vec set, %d distinct layers cycled" % n13,
+                "algorithmic_bytes_per_step": s13["total"], "floor_us_at_8TBps": round(s13["total"] / 8e6, 2)}
+        graph = capture(lambda i: [f(L13[i % n13]) for f in (qkv13, o13, sw13, dn13)], n13)
+        us, spread, replays = measure(graph, n13, replays=4 * MIN_REPLAYS)
+        capi.call("llama2_graph_destroy", graph)
+        cfg2["set"] = {"us": round(us, 3), "us_p10_median_p90": spread, "steps": replays * n13,
+                       "GBps": round(s13["total"] / us / 1e3, 1),
+                       "frac_of_hbm_peak": round(s13["total"] / us / 1e3 / HBM_PEAK_GBPS, 4)}
+        log("  cfg2 13B layer set %6.2f us  %6.0f GB/s (%.1f%% of peak; floor %.1f us)" %
+            (us, s13["total"] / us / 1e3, 100 * s13["total"] / us / 1e3 / HBM_PEAK_GBPS, s13["total"] / 8e6))
+        for name, fn in (("qkv", qkv13), ("o", o13), ("swiglu", sw13), ("down", dn13)):
+            graph = capture(lambda i, fn=fn: fn(L13[i % n13]), n13)
+            us, spread, replays = measure(graph, n13, replays=4 * MIN_REPLAYS)
+            capi.call("llama2_graph_destroy", graph)
+            cfg2[name] = {"us": round(us, 3), "us_p10_median_p90": spread, "bytes": s13[name],
+                          "GBps": round(s13[name] / us / 1e3, 1),
+                          "frac_of_hbm_peak": round(s13[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
+            log("    13B %-7s %8.2f us  %7.0f GB/s" % (name, us, s13[name] / us / 1e3))
+        result["cfg2"] = cfg2
+        for L in L13:
+            for w in L.values():
+                for b in (w.Weight, w.Zeros, w.Scales):
+                    b.free()
 
     if "calib" in legs:
         # a plain copy of known size: what FETCH_SIZE / WRITE_SIZE read for it scales the counters
@@ -278,14 +383,45 @@ def main():
             for name, fn in (("modules", modules), ("fused", fused)):
                 fn(0)  # sizes the library's scratch before capture
                 graph = capture(fn, n_layers)
-                capi.call("llama2_graph_launch", graph)
-                us = 1e3 * timed_replays(graph, 10) / (10 * n_layers)
+                us, spread, replays = measure(graph, n_layers)
                 capi.call("llama2_graph_destroy", graph)
-                row[name] = {"us": round(us, 2), "GBps": round(nbytes / us / 1e3, 1)}
+                row[name] = {"us": round(us, 2), "us_p10_median_p90": spread, "launches": replays * n_layers,
+                             "GBps": round(nbytes / us / 1e3, 1)}
             attn["S=%d" % S] = row
             log("  attention S=%-5d rope+scores+softmax+vecmat %7.2f us %6.0f GB/s | rope+fused %7.2f us %6.0f GB/s" %
                 (S, row["modules"]["us"], row["modules"]["GBps"], row["fused"]["us"], row["fused"]["GBps"]))
         result["attention"] = attn
+
+    if "chain" in legs:
+        # The whole-step persistent kernel (one launch per token, vectors handed over between workgroups as
+        # tagged words) on the same weights: its mat-vec chain (32 layers, attention skipped) per layer, and
+        # the full greedy decode through it.  Reported beside the launch sequence; the faster one is the default.
+        dec = C.c_void_p()
+        pmode = capi.DECODE_FUSED | capi.DECODE_PERSISTENT | capi.DECODE_GRAPH
+        capi.call("llama2_decode_create", C.byref(dec), C.byref(model.config), C.byref(model._w_struct),
+                  C.byref(model._s_struct), pmode)
+        graph = capture(lambda i: capi.call("llama2_decode_matvec_chain", dec, xb.ptr, x.ptr), 1)
+        us, spread, replays = measure(graph, n_layers)
+        capi.call("llama2_graph_destroy", graph)
+        capi.call("llama2_decode_check", dec)
+        n_prompt, n_gen = 128, 256
+        steps = n_prompt + n_gen - 1
+        prompt = synth.rng_for(5).integers(3, cfg["vocab_size"], n_prompt).astype(np.int32)
+        model.runstate.tokens.copy_to_device(prompt)
+        capi.call("llama2_decode_run", dec, 0, 16, n_prompt)
+        capi.call("llama2_sync")
+        ev.start()
+        capi.call("llama2_decode_run", dec, 0, steps, n_prompt)
+        ms = ev.stop_ms()
+        capi.call("llama2_decode_check", dec)
+        ptoks = model.runstate.tokens.to_host(n_prompt + n_gen)
+        result["persistent_step"] = {"matvec_chain_us_per_layer": round(us, 3), "us_p10_median_p90": spread,
+                                     "chain_launches": replays, "GBps": round(sizes["total"] / us / 1e3, 1),
+                                     "decode_tokens_per_s": round(steps / (ms * 1e-3), 1),
+                                     "last_tokens": [int(t) for t in ptoks[-4:]]}
+        log("persistent step: mat-vec chain %.2f us/layer (%.0f GB/s), decode %.1f tok/s" %
+            (us, sizes["total"] / us / 1e3, steps / (ms * 1e-3)))
+        capi.call("llama2_decode_destroy", dec)
 
     if "decode" in legs:
         # configs[4]: 128 seeded prompt tokens, 256 greedy tokens, every step on the device

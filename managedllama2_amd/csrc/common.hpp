@@ -22,6 +22,10 @@ struct Context {
     hipStream_t stream = nullptr;
     int num_cus = 0;
     bool capturing = false; // between llama2_graph_begin_capture and _end_capture
+    // A/B switches of the int4 mat-vec launches: LLAMA2_INT4_NARROW=1 one row per item for every
+    // shape, LLAMA2_INT4_BLOCKS=1 blocks of rows for every shape (default: by row length)
+    bool int4_narrow = false;
+    bool int4_blocks = false;
     // fp32 partial sums of the sequence-split attention kernels
     float* attn_partials = nullptr;
     size_t attn_partials_bytes = 0;

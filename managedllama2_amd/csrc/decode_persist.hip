@@ -33,20 +33,6 @@ constexpr int kPThreads = kPWaves * 64;
 __device__ __forceinline__ uint32_t tag16(uint32_t t) { return (t % 65535u) + 1u; } // never 0: a zeroed word is never ready
 __device__ __forceinline__ uint32_t tag32(uint32_t t) { return t | 0x80000000u; }
 
-// A pointer that is the same in every lane, moved to scalar registers.  The per-layer pointers
-// come from a table in device memory; the compiler cannot prove that nothing in this kernel writes
-// that table, loads it with vector loads, does the row arithmetic in vector registers -- and then
-// wraps every buffer load in a loop that makes its descriptor scalar again, a dozen instructions per
-// load.  One v_readfirstlane pair per descriptor avoids that.
-template <class T>
-__device__ __forceinline__ T* uniform_ptr(T* p)
-{
-    const unsigned long long v = reinterpret_cast<unsigned long long>(p);
-    const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
-    const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
-    return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
-}
-
 // One unsuccessful poll more.  Returns true when the wait has to be given up.
 __device__ __forceinline__ bool give_up(int* err, int& spins, int spin_limit)
 {
@@ -116,34 +102,6 @@ __device__ __forceinline__ float poll_part(const unsigned long long* src, uint32
     return __builtin_bit_cast(float, static_cast<uint32_t>(w));
 }
 
-// commit_pieces of int4_kernels.hpp for thread `tid` of 256 (the caller's own copy of its thread
-// number, see the layer loop): the same LDS image, the same chunk sums.
-template <int J>
-__device__ __forceinline__ void commit_pieces_t(u32x4* xs, float* sx, const VecPieces<J>& p, int tid)
-{
-    constexpr int JC = J * 64;
-#pragma unroll
-    for (int i = 0; i < J; ++i) {
-        const int e = tid + i * 256;
-        const u32x4 v = p.v[i];
-        u32x4 o;
-        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);     // x0,x4
-        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u); // x1,x5
-        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);     // x2,x6
-        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u); // x3,x7
-        xs[(e & 3) * JC + (e >> 2)] = o;
-        const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
-        float s = 0.0f;
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
-        s += dpp_f32<DPP_QUAD_XOR1>(s);
-        s += dpp_f32<DPP_QUAD_XOR2>(s);
-        if ((e & 3) == 0)
-            sx[e >> 2] = s;
-    }
-}
-
 // The first 256 threads turn the fp16 vector `raw` (LDS, K halfs) into the LDS image the int4
 // dot product reads, optionally through RMSNorm with the preloaded weights `gp`: the arithmetic
 // of the 256-thread stand-alone kernels, order included.  All threads call, with their number tid.
@@ -198,58 +156,6 @@ struct GammaPieces {
                 *reinterpret_cast<u32x4*>(gam + (tid + i * kPThreads) * 8) = v[i];
     }
 };
-
-// What a lane keeps of R rows while they are in flight: J chunks of weights per row, and -- instead
-// of one zero word and one scale per chunk -- lane l's share of the row's zero words (word l) and
-// scales (scale l + 64 k): the wavefront holds each of them once and hands them to the lanes that
-// need them when the row is computed (expand).  9 instead of 18 load instructions and 26 instead of
-// 36 registers for a row of 11008 inputs.
-template <int J, int R>
-struct CFrag {
-    static constexpr int SV = (J + 3) / 4; // 64 scales (4 chunk columns) per register
-    u32x4 w[R][J];
-    uint32_t zwv[R];
-    uint32_t sbv[R][SV];
-};
-
-// Requests row `row` of tensor m; a row that does not exist (the wavefront has no item in this
-// round) is read through buffers of zero length, which return zero and cost no traffic.  The loads
-// are unconditional on purpose: a conditional load makes the registers "old value or new value",
-// which keeps the previous round's registers alive across the whole layer.
-template <int J>
-__device__ __forceinline__ void load_row_c(u32x4 (&w)[J], uint32_t& zwv, uint32_t (&sbv)[(J + 3) / 4], const QW m, int row,
-                                           bool valid, int ws, int ss, int zs, int lane)
-{
-    const size_t r = valid ? static_cast<size_t>(row) : 0;
-    const uint32_t on = valid ? 1u : 0u;
-    const __amdgpu_buffer_rsrc_t rw = make_rsrc(uniform_ptr(m.w + r * ws), on * ws * 4);
-    const __amdgpu_buffer_rsrc_t rz = make_rsrc(uniform_ptr(m.z + r * zs), on * zs * 4);
-    const __amdgpu_buffer_rsrc_t rs = make_rsrc(uniform_ptr(m.s + r * ss), on * ss * 2);
-#pragma unroll
-    for (int j = 0; j < J; ++j)
-        w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
-    zwv = __builtin_amdgcn_raw_buffer_load_b32(rz, lane * 4, 0, 0);
-#pragma unroll
-    for (int k = 0; k < (J + 3) / 4; ++k)
-        sbv[k] = __builtin_amdgcn_raw_buffer_load_b16(rs, lane * 2 + k * 128, 0, 0);
-}
-
-// The fragment layout the dot product reads: chunk column j of lane l belongs to group
-// (l >> 2) + 16 j, whose zero point sits in zero word (l >> 5) + 2 j.
-template <int J, int R>
-__device__ __forceinline__ void expand(Frag<J, R>& f, const CFrag<J, R>& c, int lane)
-{
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-        for (int j = 0; j < J; ++j) {
-            f.w[r][j] = c.w[r][j];
-            f.zw[r][j] = static_cast<uint32_t>(
-                __builtin_amdgcn_ds_bpermute(((lane >> 5) + 2 * j) * 4, static_cast<int>(c.zwv[r])));
-            f.sb[r][j] = static_cast<uint16_t>(
-                __builtin_amdgcn_ds_bpermute((((lane >> 2) + 16 * j) & 63) * 4, static_cast<int>(c.sbv[r][j >> 2])));
-        }
-}
 
 // The per-layer pointer table is read through the constant address space: nothing writes it while
 // the kernel runs, and saying so lets the compiler fetch the pointers with scalar loads.  Read

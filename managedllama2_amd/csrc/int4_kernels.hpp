@@ -67,6 +67,9 @@ struct Int4Args {
     int kv_dim;
     float theta;
     const float* rope_table; // (cos, sin) of the step's position for i < 64, or null: computed here from theta
+#ifdef L2_PERSIST_TRACE
+    unsigned long long* trace; // diagnostic build (make TRACE=1): 16 clock readings per traced wavefront
+#endif
 };
 
 constexpr int kAuxStream = 2; // "nt": weights are touched once
@@ -321,6 +324,340 @@ __global__ __launch_bounds__(256) void int4_matvec_kernel(Int4Args a)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Blocks of consecutive rows per wavefront.
+//
+// What limits a batch-1 mat-vec on this part is neither arithmetic nor bandwidth as such but the
+// number of vector-memory INSTRUCTIONS a compute unit can have in flight (a few dozen, whatever
+// their size): a 16-byte-per-lane load carries 1 KiB, a 4- or 2-byte-per-lane load carries a
+// fraction of that and takes the same slot.  Reading a row of 4096 inputs as 2 loads of weights
+// plus 2 of zero words plus 2 of scales puts 0.35 KiB in flight per slot; a pure read achieves 1.
+// Hence:
+//   * an item is a block of RB consecutive rows: their scales are one contiguous run (RB x ss
+//     fp16, at most 256 bytes), their zero words another, so ONE 4-byte-per-lane load fetches all
+//     scales of the block and one more all zero words -- RB J + 2 slots for RB rows instead of
+//     6 J RB.  The lanes that need a scale or a zero word fetch it from the lane that holds it
+//     (ds_bpermute) when the row is computed;
+//   * the rows of a block share the reads of the staged input (dot_frag over RB rows at once);
+//   * no store between the items of a wavefront: loads and stores share one counter (vmcnt) and
+//     complete out of order with respect to each other, so after a store the compiler can only
+//     wait for "all memory operations done", the next block's loads included.  Results are
+//     collected, one per lane, and stored once;
+//   * descriptors are made scalar explicitly (uniform_ptr); a descriptor in vector registers
+//     costs a readfirstlane loop per load.
+// ---------------------------------------------------------------------------------------------
+
+// A pointer that is the same in every lane, moved to scalar registers.
+template <class T>
+__device__ __forceinline__ T* uniform_ptr(T* p)
+{
+    const unsigned long long v = reinterpret_cast<unsigned long long>(p);
+    const unsigned lo = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v));
+    const unsigned hi = __builtin_amdgcn_readfirstlane(static_cast<unsigned>(v >> 32));
+    return reinterpret_cast<T*>((static_cast<unsigned long long>(hi) << 32) | lo);
+}
+
+// What a lane keeps of R rows while they are in flight (persistent decode step): J chunks of
+// weights per row, its share of the row's zero words (word l) and of its scales (scale l + 64 k).
+template <int J, int R>
+struct CFrag {
+    static constexpr int SV = (J + 3) / 4; // 64 scales (4 chunk columns) per register
+    u32x4 w[R][J];
+    uint32_t zwv[R];
+    uint32_t sbv[R][SV];
+};
+
+// Requests row `row` of tensor m; a row that does not exist (the wavefront has no item in this
+// round) is read through buffers of zero length, which return zero and cost no traffic.
+template <int J>
+__device__ __forceinline__ void load_row_c(u32x4 (&w)[J], uint32_t& zwv, uint32_t (&sbv)[(J + 3) / 4], const QW m, int row,
+                                           bool valid, int ws, int ss, int zs, int lane)
+{
+    const size_t r = valid ? static_cast<size_t>(row) : 0;
+    const uint32_t on = valid ? 1u : 0u;
+    const __amdgpu_buffer_rsrc_t rw = make_rsrc(uniform_ptr(m.w + r * ws), on * ws * 4);
+    const __amdgpu_buffer_rsrc_t rz = make_rsrc(uniform_ptr(m.z + r * zs), on * zs * 4);
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(uniform_ptr(m.s + r * ss), on * ss * 2);
+#pragma unroll
+    for (int j = 0; j < J; ++j)
+        w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
+    zwv = __builtin_amdgcn_raw_buffer_load_b32(rz, lane * 4, 0, 0);
+#pragma unroll
+    for (int k = 0; k < (J + 3) / 4; ++k)
+        sbv[k] = __builtin_amdgcn_raw_buffer_load_b16(rs, lane * 2 + k * 128, 0, 0);
+}
+
+// The fragment layout the dot product reads: chunk column j of lane l belongs to group
+// (l >> 2) + 16 j, whose zero point sits in zero word (l >> 5) + 2 j.
+template <int J, int R>
+__device__ __forceinline__ void expand(Frag<J, R>& f, const CFrag<J, R>& c, int lane)
+{
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            f.w[r][j] = c.w[r][j];
+            f.zw[r][j] = static_cast<uint32_t>(
+                __builtin_amdgcn_ds_bpermute(((lane >> 5) + 2 * j) * 4, static_cast<int>(c.zwv[r])));
+            f.sb[r][j] = static_cast<uint16_t>(
+                __builtin_amdgcn_ds_bpermute((((lane >> 2) + 16 * j) & 63) * 4, static_cast<int>(c.sbv[r][j >> 2])));
+        }
+}
+
+// commit_pieces for thread `tid` of the first 256 of a larger workgroup.
+template <int J>
+__device__ __forceinline__ void commit_pieces_t(u32x4* xs, float* sx, const VecPieces<J>& p, int tid)
+{
+    constexpr int JC = J * 64;
+#pragma unroll
+    for (int i = 0; i < J; ++i) {
+        const int e = tid + i * 256;
+        const u32x4 v = p.v[i];
+        u32x4 o;
+        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);     // x0,x4
+        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u); // x1,x5
+        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);     // x2,x6
+        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u); // x3,x7
+        xs[(e & 3) * JC + (e >> 2)] = o;
+        const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
+        s += dpp_f32<DPP_QUAD_XOR1>(s);
+        s += dpp_f32<DPP_QUAD_XOR2>(s);
+        if ((e & 3) == 0)
+            sx[e >> 2] = s;
+    }
+}
+
+// Rows per block: what fits in 8 weight loads (32 registers) per item; RB x ss <= 128 scales
+// then always fit the one scale load (ss <= 16 J).
+constexpr int block_rows(int J, int groups) { return 8 / (J * groups) < 1 ? 1 : 8 / (J * groups); }
+
+// What a lane holds of an item: G groups (tensors, or the two halves of a RoPE pair) of RB
+// consecutive rows, J chunks each; of every group's scales the pair (2 l, 2 l + 1) of its run of
+// RB x ss, of its zero words word l of its run of RB x zs.
+template <int J, int G, int RB>
+struct BFrag {
+    u32x4 w[G][RB][J];
+    uint32_t sv[G];
+    uint32_t zv[G];
+};
+
+template <int J, int RB>
+__device__ __forceinline__ void load_block(u32x4 (&w)[RB][J], uint32_t& sv, uint32_t& zv, const QW m, int row0, int n_rows,
+                                           int ws, int ss, int zs, int lane)
+{
+    // rows [row0, row0 + RB) of a tensor with n_rows rows; rows beyond the tensor read as zero
+    const int have = n_rows - row0 < RB ? n_rows - row0 : RB;
+    const size_t r0 = static_cast<size_t>(row0);
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+        // one descriptor per row: the ragged end of a row (K not a multiple of 2048) reads as zero
+        const __amdgpu_buffer_rsrc_t rw = make_rsrc(uniform_ptr(m.w + (r0 + r) * ws), r < have ? ws * 4 : 0);
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+            w[r][j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
+    }
+    const __amdgpu_buffer_rsrc_t rs = make_rsrc(uniform_ptr(m.s + r0 * ss), have * ss * 2);
+    const __amdgpu_buffer_rsrc_t rz = make_rsrc(uniform_ptr(m.z + r0 * zs), have * zs * 4);
+    sv = __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4, 0, 0);
+    zv = __builtin_amdgcn_raw_buffer_load_b32(rz, lane * 4, 0, 0);
+}
+
+// Row r of a group in the layout the dot product reads.
+template <int J, int RB>
+__device__ __forceinline__ void expand_row(u32x4 (&fw)[J], uint32_t (&fzw)[J], uint16_t (&fsb)[J], const u32x4 (&w)[RB][J],
+                                           uint32_t sv, uint32_t zv, int r, int ss, int zs, int lane)
+{
+#pragma unroll
+    for (int j = 0; j < J; ++j) {
+        fw[j] = w[r][j];
+        const int si = r * ss + (lane >> 2) + 16 * j; // scale of group (l >> 2) + 16 j of row r
+        const uint32_t pair = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute((si >> 1) * 4, static_cast<int>(sv)));
+        fsb[j] = static_cast<uint16_t>(pair >> ((si & 1) * 16));
+        const int zi = r * zs + (lane >> 5) + 2 * j;
+        fzw[j] = static_cast<uint32_t>(__builtin_amdgcn_ds_bpermute(zi * 4, static_cast<int>(zv)));
+    }
+}
+
+template <int J, int MODE, int STAGE>
+__global__ __launch_bounds__(256) void int4_matvec_block_kernel(Int4Args a)
+{
+    constexpr int G = (MODE == SWIGLU || MODE == QKV_ROPE) ? 2 : 1; // row groups per item
+    constexpr int RB = block_rows(J, G);
+    constexpr int OUT = MODE == QKV_ROPE ? 2 * RB : RB; // results per item
+    constexpr int JC = J * 64;
+    constexpr int WAVES = 4;
+    __shared__ u32x4 xs[4 * JC];
+    __shared__ float sx[JC];
+    __shared__ float red4[4];
+    __shared__ float rope_tab[MODE == QKV_ROPE ? kRopeHeadSize : 2]; // (cos, sin) pairs
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    const int total_waves = gridDim.x * WAVES;
+    const int first_item = blockIdx.x * WAVES + wave;
+    // PLAIN / RESIDUAL / SWIGLU: blocks of RB rows per tensor; QKV_ROPE: blocks of RB (i, i + 64) pairs
+    const int per_tensor = MODE == QKV_ROPE ? (a.N >> 1) / RB : (a.N + RB - 1) / RB;
+    const int nitems = MODE == QKV_ROPE ? 3 * per_tensor : (MODE == SWIGLU ? per_tensor : a.n_tensors * per_tensor);
+
+    auto item_tensor = [&](int it) { return MODE == SWIGLU ? 0 : (it >= per_tensor) + (it >= 2 * per_tensor); };
+    auto item_row0 = [&](int it, int t) { // first row of group 0
+        const int b = it - t * per_tensor;
+        if (MODE == QKV_ROPE) {
+            const int rem = b * RB; // 64 pairs per head, 64 % RB == 0
+            return (rem >> 6) * kRopeHeadSize + (rem & 63);
+        }
+        return b * RB;
+    };
+    auto tensor = [&](int t) -> QW { return t == 0 ? a.m[0] : (t == 1 ? a.m[1] : a.m[2]); };
+    auto load_item = [&](BFrag<J, G, RB>& f, uint32_t& res, int it) {
+        it = __builtin_amdgcn_readfirstlane(it);
+        const int t = item_tensor(it), row0 = item_row0(it, t);
+        if (MODE == SWIGLU) {
+            load_block<J, RB>(f.w[0], f.sv[0], f.zv[0], a.m[0], row0, a.N, a.ws, a.ss, a.zs, lane);
+            load_block<J, RB>(f.w[G - 1], f.sv[G - 1], f.zv[G - 1], a.m[1], row0, a.N, a.ws, a.ss, a.zs, lane);
+        } else if (MODE == QKV_ROPE) {
+            load_block<J, RB>(f.w[0], f.sv[0], f.zv[0], tensor(t), row0, a.N, a.ws, a.ss, a.zs, lane);
+            load_block<J, RB>(f.w[G - 1], f.sv[G - 1], f.zv[G - 1], tensor(t), row0 + 64, a.N, a.ws, a.ss, a.zs, lane);
+        } else {
+            load_block<J, RB>(f.w[0], f.sv[0], f.zv[0], tensor(t), row0, a.N, a.ws, a.ss, a.zs, lane);
+            if (MODE == RESIDUAL) { // the residuals of the block, row r in lane r
+                const int have = a.N - row0 < RB ? a.N - row0 : RB;
+                const __amdgpu_buffer_rsrc_t ro = make_rsrc(uniform_ptr(a.out[0] + row0), have * 2);
+                res = __builtin_amdgcn_raw_buffer_load_b16(ro, lane * 2, 0, 0);
+            }
+        }
+    };
+
+    // input first (served by L2), then the first item's weights (HBM)
+    VecPieces<J> xp;
+    const uint16_t* xsrc = a.x;
+    if (STAGE == STAGE_RMSNORM && a.embedding) { // native/embedding_kernel.cu:9-11
+        int token = a.tokens[a.pos_ptr ? a.pos_ptr[0] : 0];
+        token = token < 0 ? 0 : (token >= a.vocab ? a.vocab - 1 : token); // never read outside the table
+        xsrc = a.embedding + static_cast<size_t>(token) * a.K;
+    }
+    xp.load(xsrc, a.K);
+    VecPieces<J> gp;
+    if (STAGE == STAGE_RMSNORM)
+        gp.load(a.gamma, a.K);
+    // The RoPE table is requested before the weights as well: loads return in order, so a value
+    // requested after them would hold up the staging below until the first weights have arrived.
+    float rope_entry = 0.0f;
+    if (MODE == QKV_ROPE && a.rope_table && threadIdx.x < kRopeHeadSize)
+        rope_entry = a.rope_table[threadIdx.x];
+    asm volatile("" ::: "memory"); // the input stays ahead of the weights in the memory queue
+    BFrag<J, G, RB> cur;
+    uint32_t cur_res = 0;
+    int item = first_item;
+    if (item < nitems)
+        load_item(cur, cur_res, item);
+
+    // The position lives in device memory: outside layer 0 it is read only here, after the weight
+    // loads above were issued.
+    const int pos = MODE == QKV_ROPE && a.pos_ptr ? a.pos_ptr[0] : 0;
+    if (MODE == QKV_ROPE) {
+        if (a.rope_table) { // prepared by the kernel that set the position
+            if (threadIdx.x < kRopeHeadSize)
+                rope_tab[threadIdx.x] = rope_entry;
+        } else if (threadIdx.x < kRopeHeadSize / 2) {
+            float c, s;
+            rope_cos_sin(c, s, threadIdx.x, kRopeHeadSize, pos, a.theta);
+            rope_tab[2 * threadIdx.x] = c;
+            rope_tab[2 * threadIdx.x + 1] = s;
+        }
+    }
+    if (STAGE == STAGE_RMSNORM) {
+        if (a.embedding && blockIdx.x == 0) { // the residual stream starts as the embedding row
+            const __amdgpu_buffer_rsrc_t ro = make_rsrc(a.x_out, a.K * 2);
+#pragma unroll
+            for (int i = 0; i < J; ++i)
+                __builtin_amdgcn_raw_buffer_store_b128(xp.v[i], ro, (threadIdx.x + i * 256) * 16, 0, 0);
+        }
+        const float ss = block256_sum(xp.sum_squares(), red4);
+        const float rms = 1.0f / sqrtf(ss / static_cast<float>(a.K) + a.eps); // native/rmsnorm_kernel.cu:25-27
+        xp.scale(rms, gp);
+    }
+    commit_pieces<J>(xs, sx, xp);
+    __syncthreads();
+
+    const int zshift = ((lane >> 2) & 7) * 4; // nibble of the zero word: group (c/4) % 8, same for every j
+    uint32_t outw = 0; // result p of this wavefront in lane p: item k contributes lanes [k OUT, (k + 1) OUT)
+    int filled = 0, flushed_items = 0;
+
+    // Stores what has been collected: lane p holds result p % OUT of item first_item + (flushed_items + p / OUT) total_waves.
+    auto flush = [&]() {
+        const int k = lane / OUT, o = lane - k * OUT;
+        const int it = first_item + (flushed_items + k) * total_waves;
+        if (lane < filled && it < nitems) {
+            const int t = item_tensor(it), row0 = item_row0(it, t);
+            if (MODE == QKV_ROPE) {
+                uint16_t* dst = t == 0 ? a.out[0] : (t == 1 ? a.out[1] : a.out[2]) + static_cast<size_t>(pos) * a.kv_dim;
+                const int row = row0 + (o % RB) + 64 * (o / RB);
+                dst[row] = static_cast<uint16_t>(outw);
+            } else {
+                uint16_t* dst = t == 0 ? a.out[0] : (t == 1 ? a.out[1] : a.out[2]);
+                if (row0 + o < a.N)
+                    dst[row0 + o] = static_cast<uint16_t>(outw);
+            }
+        }
+        flushed_items += filled / OUT;
+        filled = 0;
+    };
+
+    while (item < nitems) {
+        const int nitem = item + total_waves;
+        BFrag<J, G, RB> nxt;
+        uint32_t nxt_res = 0;
+        if (nitem < nitems)
+            load_item(nxt, nxt_res, nitem);
+        // the RB rows of the block (and of its partner group) against the staged input, together
+        Frag<J, G * RB> f;
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int r = 0; r < RB; ++r)
+                expand_row<J, RB>(f.w[g * RB + r], f.zw[g * RB + r], f.sb[g * RB + r], cur.w[g], cur.sv[g], cur.zv[g], r, a.ss,
+                                  a.zs, lane);
+        float acc[G * RB];
+        dot_frag<J, G * RB>(acc, f, xs, sx, lane, zshift);
+        const int t = item_tensor(item);
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+            if (MODE == SWIGLU) {
+                const float g = wave_sum(acc[r]), u = wave_sum(acc[RB + r]);
+                float v = g;
+                v *= 1.0f / (1.0f + expf(-v)); // native/mat_vec_kernel.cu:219-221
+                v *= u;
+                outw = lane == filled + r ? float_to_half_bits(v) : outw;
+            } else if (MODE == QKV_ROPE) {
+                // the unfused path stores q/k as fp16 and RoPE reads them back: keep that rounding
+                const float v0 = half_bits_to_float(float_to_half_bits(wave_sum(acc[r])));
+                const float v1 = half_bits_to_float(float_to_half_bits(wave_sum(acc[RB + r])));
+                const int i = ((item - t * per_tensor) * RB + r) & 63;
+                uint16_t b0 = float_to_half_bits(v0), b1 = float_to_half_bits(v1);
+                if (t < 2) // native/rope_kernel.cu:14-26
+                    rope_rotate(b0, b1, v0, v1, rope_tab[2 * i], rope_tab[2 * i + 1]);
+                outw = lane == filled + r ? b0 : outw;
+                outw = lane == filled + RB + r ? b1 : outw;
+            } else {
+                float v = wave_sum(acc[r]);
+                if (MODE == RESIDUAL)
+                    v += half_bits_to_float(static_cast<uint16_t>(__builtin_amdgcn_readlane(static_cast<int>(cur_res), r)));
+                outw = lane == filled + r ? float_to_half_bits(v) : outw;
+            }
+        }
+        filled += OUT;
+        if (filled + OUT > 64)
+            flush();
+        cur = nxt;
+        cur_res = nxt_res;
+        item = nitem;
+    }
+    flush();
+}
+
 // Any K (fallback beyond 8 chunk-columns per lane): runtime trip count, dynamic LDS.
 template <int MODE>
 __global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
@@ -404,11 +741,21 @@ __global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
 template <int J, int MODE, int STAGE>
 inline void launch_j(const Int4Args& a, int max_waves)
 {
-    const int nitems = MODE == QKV_ROPE ? 3 * (a.N / 2) : a.n_tensors * a.N;
-    // (giving every wavefront the same number of items -- fewer wavefronts -- measured slower: the
-    // bytes in flight matter more than the last round being half empty)
+    // Rows of up to 6144 inputs (J <= 3) measured faster one row per item (more wavefronts, each with
+    // one row in flight): 7.0 against 7.8 us for the 7B QKV launch, 10.1 against 11.7 us for SwiGLU;
+    // longer rows faster in blocks with the shared scale and zero loads (down-proj 7.4 against 7.8 us).
+    if (ctx().int4_narrow || (J <= 3 && !ctx().int4_blocks)) {
+        const int nitems = MODE == QKV_ROPE ? 3 * (a.N / 2) : a.n_tensors * a.N;
+        const int waves = nitems < max_waves ? nitems : max_waves;
+        hipLaunchKernelGGL((int4_matvec_kernel<J, MODE, STAGE>), dim3(ceil_div(waves, 4)), dim3(256), 0, ctx().stream, a);
+        return;
+    }
+    constexpr int G = (MODE == SWIGLU || MODE == QKV_ROPE) ? 2 : 1;
+    constexpr int RB = block_rows(J, G);
+    const int per_tensor = MODE == QKV_ROPE ? (a.N / 2) / RB : ceil_div(a.N, RB);
+    const int nitems = MODE == QKV_ROPE ? 3 * per_tensor : (MODE == SWIGLU ? per_tensor : a.n_tensors * per_tensor);
     const int waves = nitems < max_waves ? nitems : max_waves;
-    hipLaunchKernelGGL((int4_matvec_kernel<J, MODE, STAGE>), dim3(ceil_div(waves, 4)), dim3(256), 0, ctx().stream, a);
+    hipLaunchKernelGGL((int4_matvec_block_kernel<J, MODE, STAGE>), dim3(ceil_div(waves, 4)), dim3(256), 0, ctx().stream, a);
 }
 
 // Number of chunk-columns a lane holds per row for a K-input tensor.

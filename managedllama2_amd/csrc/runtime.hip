@@ -4,6 +4,7 @@
 #include "common.hpp"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 namespace l2 {
@@ -108,6 +109,8 @@ int llama2_init(int device)
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_keys), LLAMA2_MAX_SAMPLER_SIZE * sizeof(uint16_t)));
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_values), LLAMA2_MAX_SAMPLER_SIZE * sizeof(int)));
     c.device = device;
+    c.int4_narrow = getenv("LLAMA2_INT4_NARROW") != nullptr;
+    c.int4_blocks = getenv("LLAMA2_INT4_BLOCKS") != nullptr;
     c.ready = true;
     g_err[0] = 0;
     return LLAMA2_OK;
