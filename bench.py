@@ -379,8 +379,13 @@ def main():
                 capi.call("llama2_multi_head_attention", rs.xb.ptr, rs.q.ptr, rs.keyCache.offset_pointer(lo),
                           rs.valueCache.offset_pointer(lo), hs, dim, S, scale, heads)
 
+            def one_launch(i, S=S):
+                lo = (i % n_layers) * seq_cap * dim
+                capi.call("llama2_rope_multi_head_attention", rs.xb.ptr, rs.q.ptr, rs.keyCache.offset_pointer(lo),
+                          rs.valueCache.offset_pointer(lo), hs, dim, S, scale, heads, S, 10000.0)
+
             row = {"bytes": nbytes}
-            for name, fn in (("modules", modules), ("fused", fused)):
+            for name, fn in (("modules", modules), ("fused", fused), ("one_launch", one_launch)):
                 fn(0)  # sizes the library's scratch before capture
                 graph = capture(fn, n_layers)
                 us, spread, replays = measure(graph, n_layers)
@@ -388,8 +393,10 @@ def main():
                 row[name] = {"us": round(us, 2), "us_p10_median_p90": spread, "launches": replays * n_layers,
                              "GBps": round(nbytes / us / 1e3, 1)}
             attn["S=%d" % S] = row
-            log("  attention S=%-5d rope+scores+softmax+vecmat %7.2f us %6.0f GB/s | rope+fused %7.2f us %6.0f GB/s" %
-                (S, row["modules"]["us"], row["modules"]["GBps"], row["fused"]["us"], row["fused"]["GBps"]))
+            log("  attention S=%-5d rope+scores+softmax+vecmat %7.2f us %6.0f GB/s | rope+fused %7.2f us %6.0f GB/s | "
+                "one launch %7.2f us %6.0f GB/s" %
+                (S, row["modules"]["us"], row["modules"]["GBps"], row["fused"]["us"], row["fused"]["GBps"],
+                 row["one_launch"]["us"], row["one_launch"]["GBps"]))
         result["attention"] = attn
 
     if "chain" in legs:

@@ -98,8 +98,7 @@ int llama2_event_destroy(void* event);
  * reference, which pays one cuLaunchKernel per module call, src/Module.cs:21-22).
  * Only kernel entry points may be called while capturing: no malloc / free /
  * memcpy / sync, and llama2_vec_mat / llama2_multi_head_attention only for
- * shapes whose scratch already exists (call them once eagerly first, or use
- * llama2_multi_head_attention_static).  The captured calls keep the argument
+ * shapes whose scratch already exists (call them once eagerly first).  The captured calls keep the argument
  * values they were made with, the scratch address included: the library never
  * frees a scratch buffer before llama2_shutdown, so a later eager call that
  * needs a larger one leaves earlier graphs valid. */
@@ -195,23 +194,19 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
                                 const llama2_half* value, int head_size, int dim, int seq_length,
                                 float scale, int n_heads);
 
-/* llama2_multi_head_attention for callers that cannot allocate device memory
- * (code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc).  It has no counterpart in the reference.  Same arguments, same
- * kernels and bit-identical results; the partial results of the blocks a long
- * sequence is split into go to a fixed array inside the library (about 2.1 MB
- * per GPU, held until the process ends) instead of a buffer that grows on
- * demand, so the call never allocates or frees.  Limit: n_heads times the
- * number of blocks (128 rows each up to 3072 rows, 512 rows beyond) must not
- * exceed LLAMA2_STATIC_ATTENTION_BLOCKS, else LLAMA2_ERR_UNSUPPORTED.  Every
- * call on a GPU shares that GPU's array: calls are ordered on the library's
- * one stream; a caller that replays captured graphs of this call on streams
- * of its own must not let two of them overlap. */
-#define LLAMA2_STATIC_ATTENTION_BLOCKS 4096
-int llama2_multi_head_attention_static(llama2_half* output, const llama2_half* query,
-                                       const llama2_half* key, const llama2_half* value,
-                                       int head_size, int dim, int seq_length, float scale,
-                                       int n_heads);
+/* RoPERotation.Forward (src/RoPERotation.cs:13-21, native/rope_kernel.cu:3-26)
+ * at position `pos` followed by MultiHeadAttention (src/Transformer.cs:172-175)
+ * in ONE launch: the query and row seq_length - 1 of `key` (the row the step's
+ * QKVMatVec has just written) are rotated inside the attention kernel and
+ * written back rotated, as llama2_rope leaves them, so the call equals
+ * llama2_rope(query, key + (seq_length - 1) * dim, n_heads, 128, pos, theta,
+ * n_heads) + llama2_multi_head_attention(...) bit for bit, without the second
+ * launch.  No counterpart in the reference, which launches four kernels here.
+ * Same limits as llama2_multi_head_attention (head_size 128). */
+int llama2_rope_multi_head_attention(llama2_half* output, llama2_half* query, llama2_half* key,
+                                     const llama2_half* value, int head_size, int dim,
+                                     int seq_length, float scale, int n_heads, int pos,
+                                     float theta);
 
 /* ------------------------------------------------------- pointwise modules */
 

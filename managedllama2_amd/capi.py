@@ -16,7 +16,6 @@ ERR_NO_DEVICE = -4
 ERR_STEP_FAILED = -5
 MAX_SOFTMAX_SIZE = 8192
 MAX_SAMPLER_SIZE = 65536
-STATIC_ATTENTION_BLOCKS = 4096
 
 DECODE_MODULES = 0
 DECODE_FUSED = 1
@@ -95,7 +94,7 @@ _SIGNATURES = {
     "llama2_mat_vec_strided": [vp, vp, vp, i, i, i, i, i, i, f, i],
     "llama2_vec_mat": [vp, vp, vp, i, i, i, i, i, i],
     "llama2_multi_head_attention": [vp, vp, vp, vp, i, i, i, f, i],
-    "llama2_multi_head_attention_static": [vp, vp, vp, vp, i, i, i, f, i],
+    "llama2_rope_multi_head_attention": [vp, vp, vp, vp, i, i, i, f, i, i, f],
     "llama2_rmsnorm": [vp, vp, vp, i, f],
     "llama2_rope": [vp, vp, i, i, i, f, i],
     "llama2_softmax": [vp, i, i],

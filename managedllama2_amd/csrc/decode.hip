@@ -92,9 +92,41 @@ struct AttnArgs {
     int dim;
     int max_splits;
     float scale;
+    // ROPE variant only: the rotation of native/rope_kernel.cu:3-26 at position rope_pos is applied to
+    // the query and to row S - 1 of the key cache inside the launch, and both are written back rotated
+    uint16_t* q_rw;
+    uint16_t* k_rw;
+    int rope_pos;
+    float theta;
 };
 
-template <int WAVES>
+// Rotates the 8 elements a lane holds of a head's 128 (lane l16 of a 16-lane group: elements
+// 8 l16 .. 8 l16 + 7; the partner of element t < 64 is element t + 64, held by lane l16 ^ 8).
+__device__ __forceinline__ u32x4 rope_lane8(u32x4 mine, int l16, const float* tab /* LDS: (cos, sin) of t < 64 */)
+{
+    u32x4 other, r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+        other[k] = static_cast<uint32_t>(__shfl_xor(static_cast<int>(mine[k]), 8, 64));
+    const bool low = l16 < 8;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        uint32_t packed = 0;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int t = (l16 & 7) * 8 + 2 * k + e;
+            const uint16_t m = static_cast<uint16_t>(mine[k] >> (16 * e)), o = static_cast<uint16_t>(other[k] >> (16 * e));
+            const float v0 = half_bits_to_float(low ? m : o), v1 = half_bits_to_float(low ? o : m);
+            uint16_t b0, b1;
+            rope_rotate(b0, b1, v0, v1, tab[2 * t], tab[2 * t + 1]);
+            packed |= static_cast<uint32_t>(low ? b0 : b1) << (16 * e);
+        }
+        r[k] = packed;
+    }
+    return r;
+}
+
+template <int WAVES, bool ROPE>
 __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
 {
     constexpr int GROUPS = WAVES * 4;   // 16-lane groups, one timestep each per pass
@@ -115,7 +147,7 @@ __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
 
     const uint32_t cache_bytes = static_cast<uint32_t>(t1) * a.dim * 2; // rows of this block only; < 2^31: checked on the host
     const __amdgpu_buffer_rsrc_t rk = make_rsrc(a.kcache, cache_bytes), rv = make_rsrc(a.vcache, cache_bytes);
-    const u32x4 qv = *reinterpret_cast<const u32x4*>(a.q + col);
+    u32x4 qv = *reinterpret_cast<const u32x4*>(a.q + col);
     u32x4 kv[8], vv[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
@@ -125,6 +157,27 @@ __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
     for (int i = 0; i < 8; ++i)
         vv[i] = __builtin_amdgcn_raw_buffer_load_b128(rv, ((t0 + i * GROUPS + grp) * a.dim + col) * 2, 0,
                                                       kAuxNonTemporal);
+    if constexpr (ROPE) {
+        // the angles while the cache rows are on their way; every block of a head rotates the query
+        // for itself (in registers), the block that holds row S - 1 rotates that row and stores it
+        __shared__ float rope_tab[kRopeHeadSize];
+        if (threadIdx.x < kRopeHeadSize / 2) {
+            float c, sn;
+            rope_cos_sin(c, sn, threadIdx.x, kRopeHeadSize, a.rope_pos, a.theta);
+            rope_tab[2 * threadIdx.x] = c;
+            rope_tab[2 * threadIdx.x + 1] = sn;
+        }
+        __syncthreads();
+        qv = rope_lane8(qv, l16, rope_tab);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int row = t0 + i * GROUPS + grp;
+            if (row == S - 1) { // the same for the 16 lanes of a group
+                kv[i] = rope_lane8(kv[i], l16, rope_tab);
+                *reinterpret_cast<u32x4*>(a.k_rw + static_cast<size_t>(row) * a.dim + col) = kv[i];
+            }
+        }
+    }
     float s[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -183,6 +236,10 @@ __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
     if (nsplit == 1) {
         if (threadIdx.x < kRopeHeadSize)
             out[threadIdx.x] = float_to_half_bits(val / l);
+        if constexpr (ROPE) { // the only block of the head: all its wavefronts used the query before the barriers above
+            if (threadIdx.x < 16)
+                *reinterpret_cast<u32x4*>(a.q_rw + col) = qv;
+        }
         return;
     }
     float* P = a.part + (static_cast<size_t>(h) * a.max_splits + split) * kPartStride;
@@ -201,6 +258,11 @@ __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
         return;
     if (threadIdx.x == 0)
         store_agent(&a.counters[h], 0u); // ready for the next launch
+    if constexpr (ROPE) {
+        // every other block of the head read the query before it announced its partials
+        if (threadIdx.x < 16)
+            *reinterpret_cast<u32x4*>(a.q_rw + col) = qv;
+    }
     // Merge the blocks of this head.  The partials are read with agent-scope
     // buffer loads (they were written by other workgroups of this launch); a read
     // beyond the last block returns 0, so the loads are unconditional, and the
@@ -251,10 +313,17 @@ __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
 void launch_attn(const AttnShape& shape, int n_heads, const AttnArgs& a)
 {
     const dim3 grid(shape.splits, n_heads), block(shape.waves * 64);
+    if (a.q_rw) {
+        if (shape.waves == kSmallWaves)
+            hipLaunchKernelGGL((fused_attn_kernel<kSmallWaves, true>), grid, block, 0, ctx().stream, a);
+        else
+            hipLaunchKernelGGL((fused_attn_kernel<kAttnWaves, true>), grid, block, 0, ctx().stream, a);
+        return;
+    }
     if (shape.waves == kSmallWaves)
-        hipLaunchKernelGGL(fused_attn_kernel<kSmallWaves>, grid, block, 0, ctx().stream, a);
+        hipLaunchKernelGGL((fused_attn_kernel<kSmallWaves, false>), grid, block, 0, ctx().stream, a);
     else
-        hipLaunchKernelGGL(fused_attn_kernel<kAttnWaves>, grid, block, 0, ctx().stream, a);
+        hipLaunchKernelGGL((fused_attn_kernel<kAttnWaves, false>), grid, block, 0, ctx().stream, a);
 }
 
 // ---------------------------------------------------------------- step state
@@ -717,68 +786,6 @@ int check_attention(const char* fn, const void* output, const void* query, const
 
 } // namespace
 
-// ---------------------------------------------------------------- static scratch
-// llama2_multi_head_attention_static allocates nothing: the partial results of the
-// blocks of a head and the heads' arrival counters live in this file-scope device
-// array (one copy per GPU, at its own address, for the life of the process).  In host
-// code the array's name is only a stand-in; its device address is asked for once per
-// device, at the entry point's first call there, and every later use goes through that
-// pointer.
-namespace l2 {
-struct StaticAttnScratch {
-    float part[static_cast<size_t>(LLAMA2_STATIC_ATTENTION_BLOCKS) * kPartStride];
-    unsigned counters[kMaxAttnHeads];
-};
-} // namespace l2
-static __device__ __align__(256) unsigned char scratch[sizeof(l2::StaticAttnScratch)];
-
-namespace l2 {
-constexpr int kMaxDevices = 64;
-static StaticAttnScratch* g_static_scratch[kMaxDevices] = {};
-
-static StaticAttnScratch* static_scratch_of(int device)
-{
-    return device >= 0 && device < kMaxDevices ? g_static_scratch[device] : nullptr;
-}
-
-__global__ void clear_words_kernel(unsigned* p, int n)
-{
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n)
-        p[i] = 0u;
-}
-
-// Resolves the current device's copy of the array, once per device: asks the runtime for the
-// symbol's device address, makes sure that the runtime knows that address as device memory of this
-// device that covers the whole array (a wrong address must fail here, on the host, never in a
-// kernel), and clears the arrival counters (the kernels leave them at zero after every launch).
-int resolve_static_scratch(int device)
-{
-    if (device < 0 || device >= kMaxDevices)
-        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "device %d beyond the %d the static scratch tracks", device, kMaxDevices);
-    if (g_static_scratch[device])
-        return LLAMA2_OK;
-    void* ptr = nullptr;
-    L2_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-    size_t bytes = 0;
-    L2_HIP(hipGetSymbolSize(&bytes, HIP_SYMBOL(scratch)));
-    if (!ptr || bytes != sizeof(StaticAttnScratch))
-        return fail(LLAMA2_ERR_NO_DEVICE, "the static scratch resolves to %p, %zu bytes on device %d (expected %zu bytes)",
-                    ptr, bytes, device, sizeof(StaticAttnScratch));
-    hipPointerAttribute_t attr{};
-    L2_HIP(hipPointerGetAttributes(&attr, ptr));
-    if (attr.type != hipMemoryTypeDevice || attr.device != device || attr.devicePointer != ptr)
-        return fail(LLAMA2_ERR_NO_DEVICE, "the static scratch address %p is not device memory of device %d (type %d, device %d)",
-                    ptr, device, static_cast<int>(attr.type), attr.device);
-    StaticAttnScratch* sp = static_cast<StaticAttnScratch*>(ptr);
-    hipLaunchKernelGGL(clear_words_kernel, dim3(ceil_div(kMaxAttnHeads, 256)), dim3(256), 0, ctx().stream, sp->counters,
-                       kMaxAttnHeads);
-    L2_LAUNCH_CHECK("clear_words_kernel");
-    g_static_scratch[device] = sp;
-    return LLAMA2_OK;
-}
-} // namespace l2
-
 extern "C" {
 
 int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, const llama2_half* key,
@@ -800,29 +807,24 @@ int llama2_multi_head_attention(llama2_half* output, const llama2_half* query, c
     return LLAMA2_OK;
 }
 
-int llama2_multi_head_attention_static(llama2_half* output, const llama2_half* query, const llama2_half* key,
-                                       const llama2_half* value, int head_size, int dim, int seq_length,
-                                       float scale, int n_heads)
+int llama2_rope_multi_head_attention(llama2_half* output, llama2_half* query, llama2_half* key,
+                                     const llama2_half* value, int head_size, int dim, int seq_length, float scale,
+                                     int n_heads, int pos, float theta)
 {
     L2_REQUIRE_INIT();
-    const char* fn = "llama2_multi_head_attention_static";
+    const char* fn = "llama2_rope_multi_head_attention";
     AttnShape shape{};
     L2_TRY(check_attention(fn, output, query, key, value, head_size, dim, seq_length, n_heads, &shape));
-    StaticAttnScratch* sp = static_scratch_of(ctx().device);
-    if (!sp) { // first call on this device
-        L2_CHECK(!ctx().capturing, "%s: call it once eagerly before capturing it into a graph", fn);
-        L2_TRY(resolve_static_scratch(ctx().device));
-        sp = static_scratch_of(ctx().device);
-    }
-    if (static_cast<long long>(n_heads) * shape.splits > LLAMA2_STATIC_ATTENTION_BLOCKS)
-        return fail(LLAMA2_ERR_UNSUPPORTED,
-                    "%s: n_heads=%d x %d blocks of %d rows exceed the static scratch of %d (head, block) pairs; "
-                    "use llama2_multi_head_attention",
-                    fn, n_heads, shape.splits, shape.waves * 32, LLAMA2_STATIC_ATTENTION_BLOCKS);
+    L2_CHECK(pos >= 0, "%s: pos=%d is negative", fn, pos);
+    L2_CHECK(!overlap(output, static_cast<size_t>(n_heads) * head_size * 2, query, static_cast<size_t>(n_heads) * head_size * 2),
+             "%s: output and query overlap", fn);
+    if (shape.splits > 1)
+        L2_TRY(ensure_attn_partials(sizeof(float) * static_cast<size_t>(n_heads) * shape.splits * kPartStride));
     AttnArgs a{};
     a.q = query, a.kcache = key, a.vcache = value, a.out = output;
-    a.part = sp->part, a.counters = sp->counters, a.pos_ptr = nullptr, a.seq = seq_length;
+    a.part = ctx().attn_partials, a.counters = ctx().attn_counters, a.pos_ptr = nullptr, a.seq = seq_length;
     a.dim = dim, a.max_splits = shape.splits, a.scale = scale;
+    a.q_rw = query, a.k_rw = key, a.rope_pos = pos, a.theta = theta;
     launch_attn(shape, n_heads, a);
     L2_LAUNCH_CHECK(fn);
     return LLAMA2_OK;

@@ -6,7 +6,8 @@ import numpy as np
 from managedllama2_amd import capi, synth
 from managedllama2_amd.device import DeviceVariable, QWeight, init
 
-TOL = 2e-3  # max relative error against the fp64 dequantise-then-dot oracle
+TOL = 2e-3       # max relative error against the fp64 oracle, error floor at 2^-8 of the largest |reference|
+WORST = {}       # label -> [worst error with the 2^-8 floor, with the 2^-10 floor]; printed at the end of a run
 
 
 def up(a):
@@ -22,23 +23,30 @@ def sizes(K):
     return zs, ss, ws
 
 
-def rel_err(y, y_ref):
-    """|y - y*| / max(|y*|, 2^-8 * max|y*|).  Outputs of a zero-mean dot product
+def rel_err(y, y_ref, floor_bits=8):
+    """|y - y*| / max(|y*|, 2^-floor_bits * max|y*|).  Outputs of a zero-mean dot product
     cross zero, where a pure element-wise relative error is unbounded: an output
     that cancels to 1/1000 of its neighbours still carries the fp32 rounding
     noise of all its (up to 13824) terms.  The floor keeps the bound meaningful
     there; away from zero crossings it is the plain relative error."""
     y = np.asarray(y, np.float64)
     y_ref = np.asarray(y_ref, np.float64)
-    floor = np.max(np.abs(y_ref)) * 2.0 ** -8
+    floor = np.max(np.abs(y_ref)) * 2.0 ** -floor_bits
     return np.abs(y - y_ref) / np.maximum(np.abs(y_ref), max(floor, 1e-30))
 
 
-def assert_close(y, y_ref, what="", tol=TOL):
-    e = rel_err(y, y_ref)
-    worst = int(np.argmax(e))
-    assert e[worst] <= tol, "%s: max rel err %.3e at %d (got %r want %r)" % (
-        what, e[worst], worst, np.asarray(y).ravel()[worst], np.asarray(y_ref).ravel()[worst])
+def assert_close(y, y_ref, what="", tol=TOL, tol_fine=None):
+    """Both floors are asserted: `tol` with the 2^-8 floor, and with the 2^-10 floor `tol_fine`
+    (2 x tol unless given; the largest value measured over the whole suite is 2.4e-3, on the
+    11008-term down-projection)."""
+    tol_fine = 2 * tol if tol_fine is None else tol_fine
+    for bits, bound, slot in ((8, tol, 0), (10, tol_fine, 1)):
+        e = rel_err(y, y_ref, bits)
+        worst = int(np.argmax(e))
+        rec = WORST.setdefault(what.split(" ")[0] if what else "?", [0.0, 0.0])
+        rec[slot] = max(rec[slot], float(e[worst]))
+        assert e[worst] <= bound, "%s: max rel err %.3e (floor 2^-%d, bound %.1e) at %d (got %r want %r)" % (
+            what, e[worst], bits, bound, worst, np.asarray(y).ravel()[worst], np.asarray(y_ref).ravel()[worst])
 
 
 def ulp_diff(a, b):

@@ -4,18 +4,23 @@ embedding / classifier over a 32000 vocabulary, 128 seeded prompt tokens
 followed by 256 argmax tokens, every step on the device (hipGraph replay).
 
 The CPU oracle cannot replay 383 steps of a 7B model in test time, so it is
-teacher-forced at three positions with the GPU's own history (tokens AND
-KV-cache rows of the earlier positions): one step of the fp64 oracle is then
-compared with the GPU's logits for that step, and the GPU's token must be the
-bit-exact argmax of its logits and the oracle's argmax or a near-tie of it.
+teacher-forced at eleven positions (first, second, mid-prompt, last prompt
+token, first generated tokens, mid-generation, last) with the GPU's own history
+(tokens AND KV-cache rows of the earlier positions): one step of the fp64
+oracle is then compared with the GPU's logits for that step, and the GPU's
+token must be the bit-exact argmax of its logits and the oracle's argmax or a
+near-tie of it.  The number of positions where the two argmaxes coincide is
+printed and asserted (measured: 11 of 11; at least 10 required).
 
 Tolerance: both sides round every module output to fp16; a rounding that
-falls the other way is amplified by each of the 32 random-weight layers
-(measured: ~2e-3 of the logit range after 3 layers, ~1.4e-2 after 32), so the
-whole-model comparison is norm-wise at 3e-2.  The strict per-module bounds
-(2e-3) are enforced at these same tensor shapes in test_gpu_int4.py,
-test_gpu_f16.py, test_gpu_pointwise.py and, two layers deep, in
-test_gpu_transformer.py.
+falls the other way is amplified by each of the 32 random-weight layers.
+Measured norm-wise logit error (max |difference| / max |logit|) at the eleven
+positions: 4.3e-3, 6.0e-3, 2.4e-2, 3.3e-2, 2.5e-2, 1.4e-2, 1.2e-2, 3.2e-2,
+1.6e-2, 2.1e-2, 1.3e-2 -- it grows with the length of the attended history
+and scatters by a factor of two from position to position.  The bound is the
+largest measured value plus half: 5e-2.  The strict per-module bounds (2e-3)
+are enforced at these same tensor shapes in test_gpu_int4.py, test_gpu_f16.py,
+test_gpu_pointwise.py and, two layers deep, in test_gpu_transformer.py.
 """
 import numpy as np
 import pytest
@@ -27,7 +32,8 @@ from gpu_util import assert_close_normwise
 pytestmark = pytest.mark.gpu
 
 N_PROMPT, N_GEN = 128, 256
-DEEP_TOL = 3e-2
+DEEP_TOL = 5e-2
+MIN_EXACT = 10
 
 
 def test_full_7b_greedy_decode(oracle):
@@ -56,14 +62,15 @@ def test_full_7b_greedy_decode(oracle):
     dim, S, L = cfg["dim"], cfg["seq_len"], cfg["n_layers"]
     kc = t.runstate.keyCache.to_host().reshape(L, S, dim)
     vc = t.runstate.valueCache.to_host().reshape(L, S, dim)
-    exact = 0
-    checked = (0, N_PROMPT + 1, steps - 1)
+    exact, errs = 0, []
+    checked = (0, 1, 64, N_PROMPT - 1, N_PROMPT, N_PROMPT + 1, 200, 255, 256, 320, steps - 1)
     for pos in checked:
         hm.key_cache.reshape(L, S, dim)[:, :pos] = kc[:, :pos]
         hm.value_cache.reshape(L, S, dim)[:, :pos] = vc[:, :pos]
         want = hm.forward(pos, pos + 1).astype(np.float64)
         t.Forward(pos, pos + 1)  # rewrites row `pos` of the caches with the same values
         got = t.runstate.logits.to_host()
+        errs.append(float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want))))
         assert_close_normwise(got, want, "7B logits at pos %d" % pos, DEEP_TOL)
         tok = int(np.argmax(got))
         if pos + 1 >= N_PROMPT:
@@ -74,5 +81,7 @@ def test_full_7b_greedy_decode(oracle):
         # the step's new cache rows agree with the oracle's as well
         row = t.runstate.keyCache.to_host(dim, (L - 1) * S * dim + pos * dim).astype(np.float64)
         assert_close_normwise(row, hm.key_cache.reshape(L, S, dim)[L - 1, pos].astype(np.float64), "k row", DEEP_TOL)
-    assert exact >= 1
+    print("7B teacher-forced steps at positions %s: norm-wise logit error %s; GPU argmax == oracle argmax at %d of %d" %
+          (list(checked), ["%.2e" % e for e in errs], exact, len(checked)))
+    assert exact >= MIN_EXACT, (exact, len(checked))
     t.close()
