@@ -58,9 +58,24 @@ struct Config : llama2_config {
         std::memcpy(static_cast<llama2_config*>(&c), bytes, Size);
         if (c.rope_theta != 10000.0f) // :27-28
             throw FileLoadException("Invalid model config");
+        c.Validate();
         return c;
     }
-    int kvDim() const { return dim * n_kv_heads / n_heads; }
+    // The header comes from a file: nothing is derived from it (kvDim divides by n_heads, the sizes
+    // of the tensor stream multiply its fields) before every field is known to be sane.  The
+    // reference trusts the header and fails later with an arithmetic or a file-length exception;
+    // here a bad field is the same "Invalid model config" as a bad rope_theta.
+    void Validate() const
+    {
+        constexpr int kMaxWidth = 1 << 20, kMaxLayers = 1 << 12, kMaxVocab = 1 << 24, kMaxSeq = 1 << 24;
+        const bool ok = dim > 0 && dim <= kMaxWidth && hidden_dim > 0 && hidden_dim <= kMaxWidth && n_layers > 0 &&
+                        n_layers <= kMaxLayers && n_heads > 0 && n_heads <= dim && dim % n_heads == 0 && n_kv_heads > 0 &&
+                        n_kv_heads <= n_heads && n_heads % n_kv_heads == 0 && vocab_size > 0 && vocab_size <= kMaxVocab &&
+                        seq_len > 0 && seq_len <= kMaxSeq;
+        if (!ok)
+            throw FileLoadException("Invalid model config");
+    }
+    int kvDim() const { return static_cast<int>(static_cast<long long>(dim) * n_kv_heads / n_heads); }
 };
 static_assert(sizeof(llama2_config) == 32, "the model-file header is 32 bytes");
 

@@ -6,7 +6,8 @@ import os
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libllama2_host.so")
+# LLAMA2_HOST_LIB names another build of the facade (the sanitizer build of tests/test_oracle_sanitize.py)
+LIB_PATH = os.environ.get("LLAMA2_HOST_LIB") or os.path.join(_HERE, "libllama2_host.so")
 
 HOST_LOOP, MODULES, FUSED, FUSED_GRAPH = -1, 0, 1, 3
 _lib = None

@@ -60,6 +60,13 @@ def read_config(path):
     cfg = dict(zip(FIELDS, HEADER.unpack(raw)))
     if cfg["rope_theta"] != 10000.0:  # src/Config.cs:27-28
         raise ModelFileError("Invalid model config")
+    # nothing is derived from a header field before all of them are sane (the same limits as the C++ host layer)
+    ok = (0 < cfg["dim"] <= 1 << 20 and 0 < cfg["hidden_dim"] <= 1 << 20 and 0 < cfg["n_layers"] <= 1 << 12
+          and 0 < cfg["n_heads"] <= cfg["dim"] and cfg["dim"] % cfg["n_heads"] == 0
+          and 0 < cfg["n_kv_heads"] <= cfg["n_heads"] and cfg["n_heads"] % cfg["n_kv_heads"] == 0
+          and 0 < cfg["vocab_size"] <= 1 << 24 and 0 < cfg["seq_len"] <= 1 << 24)
+    if not ok:
+        raise ModelFileError("Invalid model config")
     return cfg
 
 

@@ -13,12 +13,13 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+# LLAMA2_ORACLE_LIB names another build of oracle.c (the sanitizer build of tests/test_oracle_sanitize.py)
+_LIB_PATH = os.environ.get("LLAMA2_ORACLE_LIB") or os.path.join(_HERE, "liboracle.so")
 
 
 def build(force=False):
     if force or not os.path.exists(_LIB_PATH):
-        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", "liboracle.so"])
+        subprocess.check_call(["make", "-C", _HERE, "-B" if force else "-s", os.path.basename(_LIB_PATH)])
     return _LIB_PATH
 
 
