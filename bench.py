@@ -38,8 +38,8 @@ sys.path.insert(0, ROOT)
 # process): (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000) x 1024.  The figure belongs to one state of the
 # kernel's source: when csrc/int4_kernels.hpp no longer hashes to the value below, the kernel has changed
 # since the counters were read and `roofline.traffic` is reported as null until they are read again.
-SWIGLU_HBM_TRAFFIC_BYTES = 47409114
-SWIGLU_HBM_TRAFFIC_SOURCE_SHA16 = "@@SHA16@@"
+SWIGLU_HBM_TRAFFIC_BYTES = 47408890
+SWIGLU_HBM_TRAFFIC_SOURCE_SHA16 = "4318338b480a4974"
 MIN_REPLAYS = 100   # graph replays behind every headline figure
 MIN_SAMPLES = 50    # replays timed one by one for the spread
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
@@ -74,9 +74,16 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline leg (0 = skip)")
     ap.add_argument("--only", default="", help="comma list of legs: set,kernel,cfg0,cfg2,calib,attn,chain,decode,sampler,repack,cpu "
                                                "(default: all but calib)")
+    ap.add_argument("--eager", action="store_true",
+                    help="issue every launch directly instead of replaying captured graphs.  For runs under rocprofv3, "
+                         "whose kernel tracing has crashed the profiled process inside hipGraphLaunch (now and then, on "
+                         "graphs of any size): the trace's per-kernel durations do not depend on how a launch was issued; "
+                         "the bench's own event timings then include the host's launch gaps and are not the ones to quote")
     ap.add_argument("--decode-mode", default="fused_graph",
                     choices=["modules", "fused", "fused_graph", "persistent", "persistent_graph"])
     args = ap.parse_args()
+    if args.eager:  # no captured graph anywhere in the process, the decoder's included
+        args.decode_mode = {"fused_graph": "fused", "persistent_graph": "persistent"}.get(args.decode_mode, args.decode_mode)
     if args.gpus != 1:
         log("bench.py: this build runs on ONE GPU (batch-1 decode has no cross-GPU exchange to measure); "
             "--gpus %d is not supported" % args.gpus)
@@ -159,8 +166,19 @@ def main():
 
     ev = Events(capi)
 
+    class Eager:
+        def __init__(self, fn, n):
+            self.fn, self.n = fn, n
+
+    def destroy(graph):
+        for g in (graph if isinstance(graph, list) else [graph]):
+            if not isinstance(g, Eager):
+                capi.call("llama2_graph_destroy", g)
+
     def capture(fn, n):
-        """Record n calls of fn(i) into one hipGraph."""
+        """Record n calls of fn(i) into one hipGraph (--eager: remember them, to be issued one by one)."""
+        if args.eager:
+            return Eager(fn, n)
         g = C.c_void_p()
         capi.call("llama2_graph_begin_capture")
         for i in range(n):
@@ -168,11 +186,22 @@ def main():
         capi.call("llama2_graph_end_capture", C.byref(g))
         return g
 
+    def launch(graph):
+        """One replay; `graph` may be a list of graphs that together make up the replay (rocprofv3's
+        kernel tracing has crashed the process inside hipGraphLaunch more often on long graphs:
+        long cycles are recorded as several graphs of 32 launches)."""
+        for g in (graph if isinstance(graph, list) else [graph]):
+            if isinstance(g, Eager):
+                for i in range(g.n):
+                    g.fn(i)
+            else:
+                capi.call("llama2_graph_launch", g)
+
     def timed_replays(graph, replays):
         capi.call("llama2_sync")
         ev.start()
         for _ in range(replays):
-            capi.call("llama2_graph_launch", graph)
+            launch(graph)
         ms = ev.stop_ms()
         capi.call("llama2_sync")
         return ms
@@ -182,12 +211,12 @@ def main():
         p10 / median / p90 over MIN_SAMPLES replays timed one by one."""
         replays = max(replays, MIN_REPLAYS)
         for _ in range(max(warmup, 1)):
-            capi.call("llama2_graph_launch", graph)
+            launch(graph)
         us = 1e3 * timed_replays(graph, replays) / (replays * units_per_replay)
         one_by_one = []
         for _ in range(MIN_SAMPLES):
             ev.start()
-            capi.call("llama2_graph_launch", graph)
+            launch(graph)
             one_by_one.append(1e3 * ev.stop_ms() / units_per_replay)
         spread = [round(float(v), 3) for v in np.percentile(np.array(one_by_one), [10, 50, 90])]
         return us, spread, replays
@@ -204,12 +233,12 @@ def main():
 
     if "set" in legs:
         # one graph = one pass over all distinct layers; K steps = K / n_layers replays, at least MIN_REPLAYS
-        graph = capture(step, n_layers)
+        graph = [capture(lambda i, lo=lo: step(lo + i), 8) for lo in range(0, n_layers, 8)]  # 4 graphs of 32 launches
         wall0 = time.perf_counter()
         us, spread, replays = measure(graph, n_layers, replays=-(-args.steps // n_layers),
                                       warmup=max(args.warmup // n_layers, 1))
         wall = time.perf_counter() - wall0
-        capi.call("llama2_graph_destroy", graph)
+        destroy(graph)
         steps = replays * n_layers
         ms_per_step = us * 1e-3
         gbps = sizes["total"] / (ms_per_step * 1e-3) / 1e9
@@ -225,7 +254,7 @@ def main():
         for name, fn in (("qkv", qkv), ("o", oproj), ("swiglu", swiglu), ("down", down)):
             graph = capture(lambda i, fn=fn: fn(layers[i % n_layers]), n_layers)
             us, spread, replays = measure(graph, n_layers)
-            capi.call("llama2_graph_destroy", graph)
+            destroy(graph)
             per_kernel[name] = {"us": round(us, 3), "us_p10_median_p90": spread, "launches": replays * n_layers,
                                 "GBps": round(sizes[name] / us / 1e3, 1), "bytes": sizes[name],
                                 "frac_of_hbm_peak": round(sizes[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
@@ -257,10 +286,12 @@ def main():
         b0 = synth.qweight_bytes(dim, dim) + 2 * dim + 2 * dim
         cfg0 = {}
         for name, entry, nbytes in (("plain", "llama2_mat_vec_int4", b0), ("residual", "llama2_mat_vec_residual_int4", b0 + 2 * dim)):
-            graph = capture(lambda i, entry=entry: capi.call(entry, x.ptr, xb.ptr, tensors[i].Weight.ptr, tensors[i].Zeros.ptr,
-                                                              tensors[i].Scales.ptr, dim, dim, zs, ss, ws), len(tensors))
-            us, spread, replays = measure(graph, len(tensors))
-            capi.call("llama2_graph_destroy", graph)
+            graphs = [capture(lambda i, entry=entry, lo=lo: capi.call(entry, x.ptr, xb.ptr, tensors[lo + i].Weight.ptr,
+                                                                       tensors[lo + i].Zeros.ptr, tensors[lo + i].Scales.ptr,
+                                                                       dim, dim, zs, ss, ws), 32)
+                      for lo in range(0, len(tensors), 32)]
+            us, spread, replays = measure(graphs, len(tensors))
+            destroy(graphs)
             cfg0[name] = {"us": round(us, 3), "us_p10_median_p90": spread, "launches": replays * len(tensors), "bytes": nbytes,
                           "GBps": round(nbytes / us / 1e3, 1), "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4),
                           "floor_us_at_8TBps": round(nbytes / 8e6, 3)}
@@ -306,7 +337,7 @@ def main():
                 "algorithmic_bytes_per_step": s13["total"], "floor_us_at_8TBps": round(s13["total"] / 8e6, 2)}
         graph = capture(lambda i: [f(L13[i % n13]) for f in (qkv13, o13, sw13, dn13)], n13)
         us, spread, replays = measure(graph, n13, replays=4 * MIN_REPLAYS)
-        capi.call("llama2_graph_destroy", graph)
+        destroy(graph)
         cfg2["set"] = {"us": round(us, 3), "us_p10_median_p90": spread, "steps": replays * n13,
                        "GBps": round(s13["total"] / us / 1e3, 1),
                        "frac_of_hbm_peak": round(s13["total"] / us / 1e3 / HBM_PEAK_GBPS, 4)}
@@ -315,7 +346,7 @@ def main():
         for name, fn in (("qkv", qkv13), ("o", o13), ("swiglu", sw13), ("down", dn13)):
             graph = capture(lambda i, fn=fn: fn(L13[i % n13]), n13)
             us, spread, replays = measure(graph, n13, replays=4 * MIN_REPLAYS)
-            capi.call("llama2_graph_destroy", graph)
+            destroy(graph)
             cfg2[name] = {"us": round(us, 3), "us_p10_median_p90": spread, "bytes": s13[name],
                           "GBps": round(s13[name] / us / 1e3, 1),
                           "frac_of_hbm_peak": round(s13[name] / us / 1e3 / HBM_PEAK_GBPS, 4)}
@@ -389,7 +420,7 @@ def main():
                 fn(0)  # sizes the library's scratch before capture
                 graph = capture(fn, n_layers)
                 us, spread, replays = measure(graph, n_layers)
-                capi.call("llama2_graph_destroy", graph)
+                destroy(graph)
                 row[name] = {"us": round(us, 2), "us_p10_median_p90": spread, "launches": replays * n_layers,
                              "GBps": round(nbytes / us / 1e3, 1)}
             attn["S=%d" % S] = row
@@ -409,7 +440,7 @@ def main():
                   C.byref(model._s_struct), pmode)
         graph = capture(lambda i: capi.call("llama2_decode_matvec_chain", dec, xb.ptr, x.ptr), 1)
         us, spread, replays = measure(graph, n_layers)
-        capi.call("llama2_graph_destroy", graph)
+        destroy(graph)
         capi.call("llama2_decode_check", dec)
         n_prompt, n_gen = 128, 256
         steps = n_prompt + n_gen - 1
@@ -488,10 +519,10 @@ def main():
             graph = capture(lambda i: (capi.call("llama2_memcpy_d2d", lg.ptr, src.ptr, vocab * 2), fn()), 16)
             base = capture(lambda i: capi.call("llama2_memcpy_d2d", lg.ptr, src.ptr, vocab * 2), 16)
             for g in (graph, base):
-                capi.call("llama2_graph_launch", g)
+                launch(g)
             us = 1e3 * (timed_replays(graph, 20) - timed_replays(base, 20)) / (20 * 16)
-            capi.call("llama2_graph_destroy", graph)
-            capi.call("llama2_graph_destroy", base)
+            destroy(graph)
+            destroy(base)
             sampler[name] = round(us, 2)
 
         timed("softmax_logits_us", lambda: capi.call("llama2_softmax_logits", lg.ptr, vocab, temp, idx.ptr))

@@ -67,9 +67,6 @@ struct Int4Args {
     int kv_dim;
     float theta;
     const float* rope_table; // (cos, sin) of the step's position for i < 64, or null: computed here from theta
-#ifdef L2_PERSIST_TRACE
-    unsigned long long* trace; // diagnostic build (make TRACE=1): 16 clock readings per traced wavefront
-#endif
 };
 
 constexpr int kAuxStream = 2; // "nt": weights are touched once

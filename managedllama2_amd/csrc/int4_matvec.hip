@@ -2,20 +2,7 @@
 // QKV, fused SwiGLU); the kernels live in int4_kernels.hpp.
 #include "int4_kernels.hpp"
 
-#include <cstdlib>
-
 namespace l2 {
-
-#ifdef L2_PERSIST_TRACE
-static unsigned long long* int4_trace()
-{
-    const char* addr = getenv("LLAMA2_INT4_TRACE"); // a device buffer of 9 x 16 64-bit words
-    return addr ? reinterpret_cast<unsigned long long*>(strtoull(addr, nullptr, 0)) : nullptr;
-}
-#define L2_SET_TRACE(a) (a).trace = int4_trace()
-#else
-#define L2_SET_TRACE(a) do { } while (0)
-#endif
 
 static int check_qweight_call(const char* fn, const void* out, const void* in, int rows, int cols,
                               int zeros_size, int scales_size, int weights_size)
@@ -69,7 +56,6 @@ int llama2_mat_vec_residual_int4(llama2_half* output, const llama2_half* input, 
     a.out[0] = output;
     a.x = input;
     a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 1;
-    L2_SET_TRACE(a);
     return launch_int4<RESIDUAL, STAGE_X>(fn, a);
 }
 
@@ -89,7 +75,6 @@ int llama2_mat_vec_int4(llama2_half* output, const llama2_half* input, const uin
     a.out[0] = output;
     a.x = input;
     a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 1;
-    L2_SET_TRACE(a);
     return launch_int4<PLAIN, STAGE_X>(fn, a);
 }
 
@@ -122,7 +107,6 @@ int llama2_qkv_mat_vec(llama2_half* q_output, llama2_half* k_output, llama2_half
     a.out[2] = v_output;
     a.x = input;
     a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 3;
-    L2_SET_TRACE(a);
     return launch_int4<PLAIN, STAGE_X>(fn, a);
 }
 
@@ -146,7 +130,6 @@ int llama2_mat_vec_swiglu(llama2_half* output, const llama2_half* input, const u
     a.out[0] = output;
     a.x = input;
     a.K = rows, a.N = cols, a.ws = weights_size, a.ss = scales_size, a.zs = zeros_size, a.n_tensors = 1;
-    L2_SET_TRACE(a);
     return launch_int4<SWIGLU, STAGE_X>(fn, a);
 }
 
