@@ -768,7 +768,8 @@ inline int launch_int4(const char* fn, const Int4Args& a)
 {
     const int J = chunk_columns(a.ws);
     const int cus = ctx().num_cus > 0 ? ctx().num_cus : 256;
-    const int short_rows = cus * ((MODE == PLAIN && a.n_tensors == 3) ? 20 : 16);
+    // 20 wavefronts per CU only where they all fit: the J = 3 kernels use 104 registers, 16 wavefronts per CU
+    const int short_rows = cus * ((MODE == PLAIN && a.n_tensors == 3 && J <= 2) ? 20 : 16);
     switch (J) {
     case 1: launch_j<1, MODE, STAGE>(a, short_rows); break;
     case 2: launch_j<2, MODE, STAGE>(a, short_rows); break;
