@@ -735,6 +735,23 @@ __global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
     }
 }
 
+// Wavefronts of a 256-thread kernel that fit on the GPU at once.  The kernels here are persistent
+// (a wavefront walks over its rows until none is left), so a grid larger than that is not "more
+// parallelism": the workgroups that do not fit start when the first ones are done, a second round
+// that nobody overlaps with (13B QKV: 13.4 us with 20 wavefronts per CU requested and 16 resident,
+// 11.0 us with 16 requested).
+template <auto Kernel>
+inline int resident_waves()
+{
+    static const int waves = [] {
+        int blocks = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, Kernel, 256, 0) != hipSuccess || blocks <= 0)
+            blocks = 2;
+        return blocks * 4 * (ctx().num_cus > 0 ? ctx().num_cus : 256);
+    }();
+    return waves;
+}
+
 template <int J, int MODE, int STAGE>
 inline void launch_j(const Int4Args& a, int max_waves)
 {
@@ -743,7 +760,9 @@ inline void launch_j(const Int4Args& a, int max_waves)
     // longer rows faster in blocks with the shared scale and zero loads (down-proj 7.4 against 7.8 us).
     if (ctx().int4_narrow || (J <= 3 && !ctx().int4_blocks)) {
         const int nitems = MODE == QKV_ROPE ? 3 * (a.N / 2) : a.n_tensors * a.N;
-        const int waves = nitems < max_waves ? nitems : max_waves;
+        const int fit = resident_waves<int4_matvec_kernel<J, MODE, STAGE>>();
+        const int cap = max_waves < fit ? max_waves : fit;
+        const int waves = nitems < cap ? nitems : cap;
         hipLaunchKernelGGL((int4_matvec_kernel<J, MODE, STAGE>), dim3(ceil_div(waves, 4)), dim3(256), 0, ctx().stream, a);
         return;
     }
@@ -751,7 +770,9 @@ inline void launch_j(const Int4Args& a, int max_waves)
     constexpr int RB = block_rows(J, G);
     const int per_tensor = MODE == QKV_ROPE ? (a.N / 2) / RB : ceil_div(a.N, RB);
     const int nitems = MODE == QKV_ROPE ? 3 * per_tensor : (MODE == SWIGLU ? per_tensor : a.n_tensors * per_tensor);
-    const int waves = nitems < max_waves ? nitems : max_waves;
+    const int fit = resident_waves<int4_matvec_block_kernel<J, MODE, STAGE>>();
+    const int cap = max_waves < fit ? max_waves : fit;
+    const int waves = nitems < cap ? nitems : cap;
     hipLaunchKernelGGL((int4_matvec_block_kernel<J, MODE, STAGE>), dim3(ceil_div(waves, 4)), dim3(256), 0, ctx().stream, a);
 }
 
@@ -768,8 +789,7 @@ inline int launch_int4(const char* fn, const Int4Args& a)
 {
     const int J = chunk_columns(a.ws);
     const int cus = ctx().num_cus > 0 ? ctx().num_cus : 256;
-    // 20 wavefronts per CU only where they all fit: the J = 3 kernels use 104 registers, 16 wavefronts per CU
-    const int short_rows = cus * ((MODE == PLAIN && a.n_tensors == 3 && J <= 2) ? 20 : 16);
+    const int short_rows = cus * ((MODE == PLAIN && a.n_tensors == 3) ? 20 : 16); // capped to what fits: launch_j
     switch (J) {
     case 1: launch_j<1, MODE, STAGE>(a, short_rows); break;
     case 2: launch_j<2, MODE, STAGE>(a, short_rows); break;
