@@ -24,8 +24,10 @@ struct Context {
     bool capturing = false; // between llama2_graph_begin_capture and _end_capture
     // A/B switches of the int4 mat-vec launches: LLAMA2_INT4_NARROW=1 one row per item for every
     // shape, LLAMA2_INT4_BLOCKS=1 blocks of rows for every shape (default: by row length)
+    // LLAMA2_INT4_NO_SPAN=1: never the span kernel (the shapes it does not take always go this way)
     bool int4_narrow = false;
     bool int4_blocks = false;
+    bool int4_no_span = false;
     // fp32 partial sums of the sequence-split attention kernels
     float* attn_partials = nullptr;
     size_t attn_partials_bytes = 0;

@@ -655,6 +655,232 @@ __global__ __launch_bounds__(256) void int4_matvec_block_kernel(Int4Args a)
     flush();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Spans of consecutive rows per wavefront, statically scheduled.
+//
+// Measured on the 7B shapes against a pure read of the same bytes (which takes 2.7 / 5.2 / 8.0 /
+// 4.7 us for the o-proj / QKV / SwiGLU / down-proj tensors), the kernels above lose their time in
+// fixed costs, not in the streaming rate:
+//   * a 2-byte result stored by 64 different workgroups into one 128-byte line, from all 8 XCDs
+//     (workgroups are dealt to the XCDs round-robin), leaves that line partially dirty in 8 L2s:
+//     0.45 us per launch at the kernel's end.  Here runs of 16 consecutive workgroups are mapped to
+//     one XCD, so a line of the output is merged in ONE L2 and written back whole;
+//   * the per-row scale / zero-word loads: a wavefront owns ROWS consecutive rows of each tensor,
+//     so their scales are one contiguous run and their zero words another, fetched once per
+//     wavefront (one or two 4-byte-per-lane loads each), parked in a wave-private piece of LDS and
+//     read per row from there.  Per row only the J 16-byte weight loads remain;
+//   * a conditional prefetch ("if there is a next row, request it") makes the compiler wait for
+//     ALL outstanding loads where the two paths merge.  Here the row sequence is fully unrolled and
+//     every load is unconditional (a row that does not exist is read through a descriptor of
+//     length zero: no traffic), so the number of loads in flight is known at every point and
+//     each wait is for exactly the loads that are needed; the staging of the input no longer
+//     waits for the first weights either;
+//   * results stay in lanes (row i of the span in lane i) and are stored once, after the last row;
+//     residual add and SwiGLU run lane-parallel there;
+//   * the first row of a span is found without a division (base / remainder from the host).
+// QKV_ROPE: a workgroup of 8 wavefronts takes rows n .. n + 3 and n + 64 .. n + 67 of a head (of
+// q, k and v), the two halves of four RoPE pairs, and exchanges the fp16-rounded results through LDS.
+// ---------------------------------------------------------------------------------------------
+
+struct SpanPlan {
+    int grid;      // workgroups
+    int base, rem; // rows per wavefront: base, one more for the first rem wavefronts
+};
+
+// Scale words (pairs of fp16) a lane fetches per tensor: ROWS rows of at most 16 J scales each.
+constexpr int span_scale_words(int J, int ROWS) { return (ROWS * 16 * J + 127) / 128; }
+
+template <int J, int MODE, int STAGE, int TN, int WAVES, int ROWS>
+__global__ __launch_bounds__(WAVES * 64) void int4_matvec_span_kernel(Int4Args a, SpanPlan plan)
+{
+    static_assert(MODE != QKV_ROPE || (WAVES == 8 && ROWS == 1 && TN == 3), "RoPE pairs: 8 wavefronts, one row each");
+    constexpr int SD = span_scale_words(J, ROWS);
+    constexpr int JC = J * 64;
+    constexpr int Q = ROWS * TN; // row loads per wavefront
+    __shared__ u32x4 xs[4 * JC];
+    __shared__ float sx[JC];
+    __shared__ float red4[4];
+    __shared__ uint32_t meta_s[WAVES][TN][SD * 64];
+    __shared__ uint32_t meta_z[WAVES][TN][64];
+    __shared__ float rope_tab[MODE == QKV_ROPE ? kRopeHeadSize : 2]; // (cos, sin) pairs
+    __shared__ float pair_val[MODE == QKV_ROPE ? 2 * WAVES : 2];     // q and k of every wavefront's row
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+    // Workgroups go to the 8 XCDs round-robin: within every aligned group of 128 workgroups, give each
+    // XCD a run of 16 consecutive ones (64 or more consecutive rows: whole lines of the output).
+    int bx = blockIdx.x;
+    if (bx < static_cast<int>(gridDim.x & ~127u)) {
+        const int k = bx >> 3;
+        bx = (k >> 4) * 128 + (bx & 7) * 16 + (k & 15);
+    }
+    int r0, n;
+    if (MODE == QKV_ROPE) { // 16 workgroups per head: rows 4 b .. 4 b + 3 (wavefronts 0-3) and + 64 (wavefronts 4-7)
+        r0 = (bx >> 4) * kRopeHeadSize + (bx & 15) * 4 + (wave & 3) + (wave >> 2) * 64;
+        n = r0 < a.N ? 1 : 0;
+    } else {
+        const int gw = bx * WAVES + wave;
+        r0 = gw * plan.base + (gw < plan.rem ? gw : plan.rem);
+        n = plan.base + (gw < plan.rem ? 1 : 0); // ROWS or ROWS - 1; 0 beyond the tensor
+        if (r0 >= a.N)
+            n = 0;
+    }
+
+    auto load_w = [&](u32x4 (&w)[J], int q) { // q = i TN + t: constants after unrolling
+        const int i = q / TN, t = q % TN;
+        const __amdgpu_buffer_rsrc_t rw =
+            make_rsrc(uniform_ptr(a.m[t].w + static_cast<size_t>(r0 + i) * a.ws), i < n ? a.ws * 4 : 0);
+#pragma unroll
+        for (int j = 0; j < J; ++j)
+            w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
+    };
+
+    // input first, then the span's scales / zero words / residuals, then the first row
+    const bool stager = WAVES == 4 || threadIdx.x < 256;
+    VecPieces<J> xp, gp;
+    const uint16_t* xsrc = a.x;
+    if (STAGE == STAGE_RMSNORM && a.embedding) { // native/embedding_kernel.cu:9-11
+        int token = a.tokens[a.pos_ptr ? a.pos_ptr[0] : 0];
+        token = token < 0 ? 0 : (token >= a.vocab ? a.vocab - 1 : token); // never read outside the table
+        xsrc = a.embedding + static_cast<size_t>(token) * a.K;
+    }
+    if (stager) {
+        xp.load(xsrc, a.K);
+        if (STAGE == STAGE_RMSNORM)
+            gp.load(a.gamma, a.K);
+    }
+    float rope_entry = 0.0f;
+    if (MODE == QKV_ROPE && a.rope_table && threadIdx.x < kRopeHeadSize)
+        rope_entry = a.rope_table[threadIdx.x];
+    uint32_t sreg[TN][SD], zreg[TN], res = 0;
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+        const __amdgpu_buffer_rsrc_t rs = make_rsrc(uniform_ptr(a.m[t].s + static_cast<size_t>(r0) * a.ss), n * a.ss * 2);
+        const __amdgpu_buffer_rsrc_t rz = make_rsrc(uniform_ptr(a.m[t].z + static_cast<size_t>(r0) * a.zs), n * a.zs * 4);
+#pragma unroll
+        for (int k = 0; k < SD; ++k)
+            sreg[t][k] = __builtin_amdgcn_raw_buffer_load_b32(rs, lane * 4 + k * 256, 0, 0);
+        zreg[t] = __builtin_amdgcn_raw_buffer_load_b32(rz, lane * 4, 0, 0);
+    }
+    if (MODE == RESIDUAL) {
+        const __amdgpu_buffer_rsrc_t ro = make_rsrc(uniform_ptr(a.out[0] + r0), n * 2);
+        res = __builtin_amdgcn_raw_buffer_load_b16(ro, lane * 2, 0, 0);
+    }
+    asm volatile("" ::: "memory"); // the small loads stay ahead of the weights in the memory queue
+    u32x4 ring[2][J];
+    load_w(ring[0], 0);
+    asm volatile("" ::: "memory");
+
+    const int pos = MODE == QKV_ROPE && a.pos_ptr ? a.pos_ptr[0] : 0;
+    if (MODE == QKV_ROPE) {
+        if (a.rope_table) { // prepared by the kernel that set the position
+            if (threadIdx.x < kRopeHeadSize)
+                rope_tab[threadIdx.x] = rope_entry;
+        } else if (threadIdx.x < kRopeHeadSize / 2) {
+            float c, sn;
+            rope_cos_sin(c, sn, threadIdx.x, kRopeHeadSize, pos, a.theta);
+            rope_tab[2 * threadIdx.x] = c;
+            rope_tab[2 * threadIdx.x + 1] = sn;
+        }
+    }
+    if (STAGE == STAGE_RMSNORM) {
+        if (a.embedding && blockIdx.x == 0 && stager) { // the residual stream starts as the embedding row
+            const __amdgpu_buffer_rsrc_t ro = make_rsrc(a.x_out, a.K * 2);
+#pragma unroll
+            for (int i = 0; i < J; ++i)
+                __builtin_amdgcn_raw_buffer_store_b128(xp.v[i], ro, (threadIdx.x + i * 256) * 16, 0, 0);
+        }
+        // the sum of the stand-alone RMSNorm: wavefronts 0-3 each a quarter, added in its order
+        float part = stager ? wave_sum(xp.sum_squares()) : 0.0f;
+        if (stager && lane == 0)
+            red4[wave] = part;
+        __syncthreads();
+        const float ss = (red4[0] + red4[1]) + (red4[2] + red4[3]);
+        const float rms = 1.0f / sqrtf(ss / static_cast<float>(a.K) + a.eps); // native/rmsnorm_kernel.cu:25-27
+        if (stager)
+            xp.scale(rms, gp);
+    }
+    if (stager)
+        commit_pieces_t<J>(xs, sx, xp, threadIdx.x);
+#pragma unroll
+    for (int t = 0; t < TN; ++t) {
+#pragma unroll
+        for (int k = 0; k < SD; ++k)
+            meta_s[wave][t][lane + 64 * k] = sreg[t][k];
+        meta_z[wave][t][lane] = zreg[t];
+    }
+    __syncthreads();
+
+    const int zshift = ((lane >> 2) & 7) * 4; // nibble of the zero word: group (c/4) % 8, same for every j
+    float outv[TN];
+#pragma unroll
+    for (int t = 0; t < TN; ++t)
+        outv[t] = 0.0f;
+#pragma unroll
+    for (int q = 0; q < Q; ++q) {
+        if (q + 1 < Q)
+            load_w(ring[(q + 1) & 1], q + 1);
+        const int i = q / TN, t = q % TN;
+        Frag<J, 1> cur;
+        const uint16_t* sp = reinterpret_cast<const uint16_t*>(&meta_s[wave][t][0]) + i * a.ss + (lane >> 2);
+        const uint32_t* zp = &meta_z[wave][t][0] + i * a.zs + (lane >> 5);
+#pragma unroll
+        for (int j = 0; j < J; ++j) {
+            cur.w[0][j] = ring[q & 1][j];
+            cur.sb[0][j] = sp[16 * j];
+            cur.zw[0][j] = zp[2 * j];
+        }
+        float acc[1];
+        dot_frag<J, 1>(acc, cur, xs, sx, lane, zshift);
+        const float s = wave_sum(acc[0]);
+        outv[t] = lane == i ? s : outv[t];
+    }
+
+    if (MODE == QKV_ROPE) {
+        // the unfused path stores q/k as fp16 and RoPE reads them back: keep that rounding
+        const float qv = half_bits_to_float(float_to_half_bits(__builtin_bit_cast(
+            float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, outv[0])))));
+        const float kv = half_bits_to_float(float_to_half_bits(__builtin_bit_cast(
+            float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, outv[TN > 1 ? 1 : 0])))));
+        if (lane == 0) {
+            pair_val[2 * wave] = qv;
+            pair_val[2 * wave + 1] = kv;
+        }
+        __syncthreads();
+        if (lane == 0 && n) {
+            const int partner = wave ^ 4, i = r0 & 63; // pair index within the head
+            const float c = rope_tab[2 * i], sn = rope_tab[2 * i + 1];
+            uint16_t* kdst = a.out[1] + static_cast<size_t>(pos) * a.kv_dim;
+            uint16_t* vdst = a.out[TN > 2 ? 2 : 0] + static_cast<size_t>(pos) * a.kv_dim;
+            uint16_t b0, b1;
+            // native/rope_kernel.cu:14-26: (v0, v1) = rows (i, i + 64) of the head
+            if (wave < 4) {
+                rope_rotate(b0, b1, qv, pair_val[2 * partner], c, sn);
+                a.out[0][r0] = b0;
+                rope_rotate(b0, b1, kv, pair_val[2 * partner + 1], c, sn);
+                kdst[r0] = b0;
+            } else {
+                rope_rotate(b0, b1, pair_val[2 * partner], qv, c, sn);
+                a.out[0][r0] = b1;
+                rope_rotate(b0, b1, pair_val[2 * partner + 1], kv, c, sn);
+                kdst[r0] = b1;
+            }
+            vdst[r0] = float_to_half_bits(outv[TN > 2 ? 2 : 0]);
+        }
+    } else if (lane < n) {
+        if (MODE == SWIGLU) {
+            float v = outv[0];
+            v *= 1.0f / (1.0f + expf(-v)); // native/mat_vec_kernel.cu:219-221
+            v *= outv[TN - 1];
+            a.out[0][r0 + lane] = float_to_half_bits(v);
+        } else if (MODE == RESIDUAL) {
+            a.out[0][r0 + lane] = float_to_half_bits(outv[0] + half_bits_to_float(static_cast<uint16_t>(res)));
+        } else {
+#pragma unroll
+            for (int t = 0; t < TN; ++t)
+                a.out[t][r0 + lane] = float_to_half_bits(outv[t]);
+        }
+    }
+}
+
 // Any K (fallback beyond 8 chunk-columns per lane): runtime trip count, dynamic LDS.
 template <int MODE>
 __global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
@@ -740,21 +966,77 @@ __global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
 // parallelism": the workgroups that do not fit start when the first ones are done, a second round
 // that nobody overlaps with (13B QKV: 13.4 us with 20 wavefronts per CU requested and 16 resident,
 // 11.0 us with 16 requested).
-template <auto Kernel>
+template <auto Kernel, int THREADS = 256>
 inline int resident_waves()
 {
-    static const int waves = [] {
+    static int waves = 0, for_cus = -1; // per kernel instantiation; recomputed if the device changed
+    const int cus = ctx().num_cus > 0 ? ctx().num_cus : 256;
+    if (for_cus != cus) {
         int blocks = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, Kernel, 256, 0) != hipSuccess || blocks <= 0)
-            blocks = 2;
-        return blocks * 4 * (ctx().num_cus > 0 ? ctx().num_cus : 256);
-    }();
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, Kernel, THREADS, 0) != hipSuccess || blocks <= 0)
+            blocks = 1;
+        waves = blocks * (THREADS / 64) * cus;
+        for_cus = cus;
+    }
     return waves;
+}
+
+// The span kernel for this launch, if the shape suits it: scales readable 4 bytes at a time, and
+// all wavefronts resident at once with ROWS rows each.
+template <int J, int MODE, int STAGE, int TN, int WAVES, int ROWS>
+inline bool try_span(const Int4Args& a)
+{
+    constexpr auto kernel = int4_matvec_span_kernel<J, MODE, STAGE, TN, WAVES, ROWS>;
+    SpanPlan plan{};
+    if (MODE == QKV_ROPE) {
+        if (a.N % kRopeHeadSize)
+            return false;
+        plan.grid = a.N / 8;
+    } else {
+        int waves = ceil_div(a.N, ROWS);
+        waves = ceil_div(waves, WAVES * 8) * (WAVES * 8);
+        plan.grid = waves / WAVES;
+        plan.base = a.N / waves, plan.rem = a.N % waves;
+    }
+    if (plan.grid * WAVES > resident_waves<kernel, WAVES * 64>())
+        return false;
+    hipLaunchKernelGGL(kernel, dim3(plan.grid), dim3(WAVES * 64), 0, ctx().stream, a, plan);
+    return true;
+}
+
+template <int J, int MODE, int STAGE>
+inline bool launch_span(const Int4Args& a)
+{
+    if (ctx().int4_no_span || ctx().int4_narrow || ctx().int4_blocks || (a.ss & 1))
+        return false;
+    const int tn = MODE == SWIGLU ? 2 : a.n_tensors;
+    for (int t = 0; t < tn; ++t)
+        if (!aligned(a.m[t].s, 4))
+            return false;
+    // Rows per wavefront and wavefronts per workgroup as measured on the 7B / 13B shapes: one row per
+    // wavefront where that many wavefronts fit, three for the SwiGLU pair of tensors.
+    if constexpr (MODE == QKV_ROPE) {
+        return a.n_tensors == 3 && try_span<J, MODE, STAGE, 3, 8, 1>(a);
+    } else if constexpr (MODE == SWIGLU) {
+        return try_span<J, MODE, STAGE, 2, 8, 3>(a) || try_span<J, MODE, STAGE, 2, 8, 4>(a);
+    } else if constexpr (MODE == PLAIN) {
+        if (a.n_tensors == 3)
+            return try_span<J, MODE, STAGE, 3, 8, 1>(a) || try_span<J, MODE, STAGE, 3, 8, 2>(a);
+        if (a.n_tensors != 1)
+            return false;
+    }
+    if constexpr (MODE == PLAIN || MODE == RESIDUAL) {
+        constexpr int W = J <= 3 ? 4 : 8;
+        return try_span<J, MODE, STAGE, 1, W, 1>(a) || try_span<J, MODE, STAGE, 1, W, 2>(a);
+    }
+    return false;
 }
 
 template <int J, int MODE, int STAGE>
 inline void launch_j(const Int4Args& a, int max_waves)
 {
+    if (launch_span<J, MODE, STAGE>(a))
+        return;
     // Rows of up to 6144 inputs (J <= 3) measured faster one row per item (more wavefronts, each with
     // one row in flight): 7.0 against 7.8 us for the 7B QKV launch, 10.1 against 11.7 us for SwiGLU;
     // longer rows faster in blocks with the shared scale and zero loads (down-proj 7.4 against 7.8 us).
