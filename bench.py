@@ -187,9 +187,7 @@ def main():
         return g
 
     def launch(graph):
-        """One replay; `graph` may be a list of graphs that together make up the replay (rocprofv3's
-        kernel tracing has crashed the process inside hipGraphLaunch more often on long graphs:
-        long cycles are recorded as several graphs of 32 launches)."""
+        """One replay (`graph` may be a list of graphs that together make up the replay)."""
         for g in (graph if isinstance(graph, list) else [graph]):
             if isinstance(g, Eager):
                 for i in range(g.n):
@@ -233,7 +231,7 @@ def main():
 
     if "set" in legs:
         # one graph = one pass over all distinct layers; K steps = K / n_layers replays, at least MIN_REPLAYS
-        graph = [capture(lambda i, lo=lo: step(lo + i), 8) for lo in range(0, n_layers, 8)]  # 4 graphs of 32 launches
+        graph = capture(step, n_layers)  # 4 launches x 32 layers in one graph
         wall0 = time.perf_counter()
         us, spread, replays = measure(graph, n_layers, replays=-(-args.steps // n_layers),
                                       warmup=max(args.warmup // n_layers, 1))
@@ -264,7 +262,7 @@ def main():
         src = os.path.join(ROOT, "managedllama2_amd", "csrc", "int4_kernels.hpp")
         sha16 = hashlib.sha256(open(src, "rb").read()).hexdigest()[:16] if os.path.exists(src) else None
         fresh = sha16 == SWIGLU_HBM_TRAFFIC_SOURCE_SHA16
-        result["roofline"] = {"bound": "hbm", "kernel": "int4_matvec_kernel<2, SWIGLU> (fused gate/up, 2x11008x4096)",
+        result["roofline"] = {"bound": "hbm", "kernel": "int4_matvec_span_kernel<2, SWIGLU, STAGE_X, 2, 8, 3> (fused gate/up, 2x11008x4096)",
                               "achieved": dom["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                               "frac": round(dom["GBps"] / HBM_PEAK_GBPS, 4),
                               "traffic": SWIGLU_HBM_TRAFFIC_BYTES if fresh else None,
@@ -286,10 +284,9 @@ def main():
         b0 = synth.qweight_bytes(dim, dim) + 2 * dim + 2 * dim
         cfg0 = {}
         for name, entry, nbytes in (("plain", "llama2_mat_vec_int4", b0), ("residual", "llama2_mat_vec_residual_int4", b0 + 2 * dim)):
-            graphs = [capture(lambda i, entry=entry, lo=lo: capi.call(entry, x.ptr, xb.ptr, tensors[lo + i].Weight.ptr,
-                                                                       tensors[lo + i].Zeros.ptr, tensors[lo + i].Scales.ptr,
-                                                                       dim, dim, zs, ss, ws), 32)
-                      for lo in range(0, len(tensors), 32)]
+            graphs = capture(lambda i, entry=entry: capi.call(entry, x.ptr, xb.ptr, tensors[i].Weight.ptr,
+                                                               tensors[i].Zeros.ptr, tensors[i].Scales.ptr,
+                                                               dim, dim, zs, ss, ws), len(tensors))
             us, spread, replays = measure(graphs, len(tensors))
             destroy(graphs)
             cfg0[name] = {"us": round(us, 3), "us_p10_median_p90": spread, "launches": replays * len(tensors), "bytes": nbytes,

@@ -369,10 +369,14 @@ typedef struct llama2_decoder llama2_decoder;
  * LLAMA2_DECODE_FUSED.  Serves histories of up to 3072 rows (longer ones fall
  * back to the launch sequence, step by step) and the shapes it has kernels for
  * (Llama-2-7B: dim 4096, hidden_dim 11008, 32 heads on 256 compute units; and
- * models up to dim 2048 / hidden_dim 2048); otherwise llama2_decode_create
+ * small models of at most one row per wavefront and phase: on 256 compute units
+ * dim <= 640 and hidden_dim <= 2048); otherwise llama2_decode_create
  * returns LLAMA2_ERR_UNSUPPORTED.  The launch needs the GPU to itself: all its
  * workgroups must be resident at once.  Every wait inside it is bounded; a step
- * that gives up raises a flag that llama2_decode_check reports. */
+ * that gives up raises a sticky flag: llama2_decode_sample and
+ * llama2_decode_sample_top_p return LLAMA2_ERR_STEP_FAILED from then on, and
+ * after the asynchronous llama2_decode_run / _run_sampled the caller asks
+ * llama2_decode_check. */
 #define LLAMA2_DECODE_PERSISTENT 4
 
 /* Binds a config, a weight set and a run state (all borrowed, all must outlive

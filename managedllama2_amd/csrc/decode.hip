@@ -331,8 +331,9 @@ void launch_attn(const AttnShape& shape, int n_heads, const AttnArgs& a)
 // state[2] = 1 to advance the position after sampling, state[3] = number of
 // token slots (the context length: the token after the last row has no slot and
 // is not stored), state[4] = a spare slot for that token when the host asks for
-// it, state[5] = a serial number that every kernel which sets or advances the
-// position increments (the persistent step derives its hand-over tags from it),
+// it, state[5] = the number of persistent steps so far, incremented by a one-thread
+// launch right before each of them and by nothing else (the persistent step derives
+// its hand-over tags from it: successive tags of a word differ by 1 .. n_layers + 2),
 // state[6] = the persistent step's error flag (persist.hpp names the indices);
 // the 128 floats behind the 8 ints hold (cos, sin) of the position's RoPE
 // angles, so the 32 QKV launches of a step do not each call powf/cosf/sinf.
@@ -354,7 +355,6 @@ __global__ void set_state_kernel(int* state, int pos, int n_prompt, int advance,
         state[1] = n_prompt;
         state[2] = advance;
         state[3] = n_slots;
-        state[kStateSerial] = state[kStateSerial] + 1;
     }
     if (threadIdx.x < kRopeHeadSize / 2)
         write_rope_table(state, threadIdx.x, pos, theta);
@@ -383,7 +383,6 @@ __global__ __launch_bounds__(1024) void argmax_step_kernel(const uint16_t* x, in
             tokens[pos0 + 1] = best;
         if (advance0)
             state[0] = pos0 + 1;
-        state[kStateSerial] = state[kStateSerial] + 1;
     }
 }
 
@@ -420,7 +419,6 @@ __device__ __forceinline__ void sample_step(const SampleStepArgs& a, SamplerLds&
     if (threadIdx.x == 0) {
         if (advance0)
             a.state[0] = pos0 + 1;
-        a.state[kStateSerial] = a.state[kStateSerial] + 1;
     }
 }
 
@@ -574,8 +572,11 @@ int persist_setup(llama2_decoder* d)
 // `shape` (attn_shape_index of an upper bound of position + 1) sizes the attention grid.
 int forward_fused(llama2_decoder* d, int shape)
 {
-    if (shape == kPersistShape) // the whole step in one launch
+    if (shape == kPersistShape) { // the whole step in one launch, behind the bump of its own step counter
+        hipLaunchKernelGGL(bump_serial_kernel, dim3(1), dim3(64), 0, ctx().stream, d->state);
+        L2_LAUNCH_CHECK("bump_serial_kernel");
         return persist_launch(d->persist_variant, d->pa, ctx().num_cus);
+    }
     const AttnShape as = attn_shape(shape, d->cfg.seq_len);
     const llama2_config& c = d->cfg;
     const llama2_run_state& s = d->s;
@@ -971,6 +972,21 @@ int llama2_decode_create(llama2_decoder** decoder, const llama2_config* config,
     return LLAMA2_OK;
 }
 
+// The persistent step's failure flag is sticky (every later wait gives up at once): wherever the
+// library hands a token back to the host, which waits for the GPU anyway, the flag comes with it.
+static int persist_status(llama2_decoder* d, const char* fn)
+{
+    if (d->persist_variant < 0)
+        return LLAMA2_OK;
+    int flag = 0;
+    L2_TRY(llama2_memcpy_d2h(&flag, d->state, static_cast<size_t>(kStateError) * sizeof(int), sizeof(int)));
+    if (flag != 0)
+        return fail(LLAMA2_ERR_STEP_FAILED,
+                    "%s: a persistent step gave up waiting for data from another workgroup; the decoder's results "
+                    "are undefined from that step on (llama2_decode_check has the details)", fn);
+    return LLAMA2_OK;
+}
+
 int llama2_decode_forward(llama2_decoder* d, int position, int next_position)
 {
     L2_REQUIRE_INIT();
@@ -995,7 +1011,8 @@ int llama2_decode_sample(llama2_decoder* d, int next_position, int generate_toke
     L2_CHECK(slot.tokens == d->s.tokens || generate_token,
              "llama2_decode_sample: next_position=%d is past the last token of the context", next_position);
     L2_TRY(llama2_argmax(d->s.logits, d->cfg.vocab_size, slot.tokens, slot.index, generate_token));
-    return llama2_memcpy_d2h(token, slot.tokens, static_cast<size_t>(slot.index) * sizeof(int), sizeof(int));
+    L2_TRY(llama2_memcpy_d2h(token, slot.tokens, static_cast<size_t>(slot.index) * sizeof(int), sizeof(int)));
+    return persist_status(d, "llama2_decode_sample");
 }
 
 int llama2_decode_sample_top_p(llama2_decoder* d, int next_position, int generate_token, float temperature,
@@ -1011,7 +1028,8 @@ int llama2_decode_sample_top_p(llama2_decoder* d, int next_position, int generat
     const TokenSlot slot = token_slot(d, next_position);
     L2_TRY(sample_launch(fn, d->s.logits, d->s.indices, d->cfg.vocab_size, temperature, top_p, coin, slot.tokens,
                          slot.index, true)); // :50-66
-    return llama2_memcpy_d2h(token, slot.tokens, static_cast<size_t>(slot.index) * sizeof(int), sizeof(int)); // :69
+    L2_TRY(llama2_memcpy_d2h(token, slot.tokens, static_cast<size_t>(slot.index) * sizeof(int), sizeof(int))); // :69
+    return persist_status(d, fn);
 }
 
 float llama2_sampler_coin(unsigned long long seed, int position) { return sampler_coin(seed, position); }

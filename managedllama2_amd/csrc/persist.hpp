@@ -23,7 +23,7 @@ constexpr int kStatePrompt = 1;   // first position whose token is generated
 constexpr int kStateAdvance = 2;  // 1: the sampling kernel advances the position
 constexpr int kStateSlots = 3;    // token slots (context length)
 constexpr int kSpareTokenSlot = 4;
-constexpr int kStateSerial = 5;   // counts steps: the hand-over tags of the persistent step derive from it
+constexpr int kStateSerial = 5;   // counts persistent steps (bumped right before each, by nothing else): their hand-over tags derive from it
 constexpr int kStateError = 6;    // set by the persistent step when a bounded wait gave up
 
 struct PersistLayer { // one per layer, in device memory

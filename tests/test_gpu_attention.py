@@ -43,6 +43,8 @@ def modules(q, k, v, dim, heads, seq):
     return out.to_host()[:heads * HS]
 
 
+MAX_TIE_FRACTION = 0.025  # of all scores may take the tie slack (measured: 1.6 .. 1.8 % at 100 .. 8192 rows)
+TIES = []   # (scores that took the tie slack, scores) of every oracle_chain(..., with_slack=True) call
 TIE = 1e-6  # a score this close to the midpoint of two fp16 values may round either way (fp32 sum of 128 products)
 
 
@@ -65,6 +67,7 @@ def oracle_chain(oracle, q, k, v, dim, heads, seq, with_slack=False):
     near = (step / 2 - np.abs(scores.reshape(heads, seq) - r)) < TIE
     w = np.where(near, p * step, 0.0)  # d p_t = p_t * d s_t
     slack = np.einsum("ht,thj->hj", w, np.abs(vv)) + w.sum(axis=1)[:, None] * np.abs(out)
+    TIES.append((int(near.sum()), near.size))
     return out.ravel(), slack.ravel()
 
 
@@ -72,6 +75,9 @@ def assert_close_up_to_ties(got, want_slack, what):
     """gpu_util.assert_close (2e-3 with the 2^-8 floor, 4e-3 with the 2^-10 floor) after taking
     the tie slack off the difference."""
     want, slack = want_slack
+    n_tie, n_scores = TIES[-1]
+    print("%s: %d of %d scores within %g of an fp16 rounding midpoint took the tie slack" % (what, n_tie, n_scores, TIE))
+    assert n_tie <= MAX_TIE_FRACTION * n_scores + 2, (what, n_tie, n_scores)
     diff = got.astype(np.float64) - want
     diff = np.sign(diff) * np.maximum(np.abs(diff) - slack, 0.0)
     assert_close(want + diff, want, what)

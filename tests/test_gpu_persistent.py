@@ -205,6 +205,10 @@ def test_wait_limit_failure_is_reported_not_hung():
         assert np.array_equal(bits(t.runstate.logits.to_host()), bits(good))
     else:
         assert rc == capi.ERR_STEP_FAILED and "gave up" in capi.last_error()
+        # the flag is sticky: the entry points that hand a token to the host report it too
+        import ctypes
+        token = ctypes.c_int()
+        assert capi.raw("llama2_decode_sample", t._decoder, 1, 1, ctypes.byref(token)) == capi.ERR_STEP_FAILED
     capi.call("llama2_decode_set_wait_limit", t._decoder, 1 << 21)
     t.Forward(0, 1)
     check_ok(t)
