@@ -97,20 +97,37 @@ __device__ __forceinline__ void load_row(u32x4 (&w)[J], uint32_t (&zw)[J], uint1
 // LDS image of the input for J chunk-columns per lane:
 //   xs[i*JC + c] holds elements 8*(4c+i)+{0,4,1,5,2,6,3,7} (JC = 64 J, zero beyond K),
 //   sx[c] the fp32 sum of the 32 elements of chunk c.
+// 8 consecutive inputs (words `word` and the three after it of a chunk's 16) in the order the nibble
+// extraction produces them: (x0,x4), (x1,x5), (x2,x6), (x3,x7).
+//
+// v_dot2_f32_f16 does not round its fp32 result to nearest: it drops what lies below about 2^-40
+// (an ABSOLUTE position, whatever the magnitude of the operands) towards minus infinity.  The sums
+// of nibble * 2^-24 * x live just above that position, and a mat-vec of 11008 terms came out low
+// by 4.0e-5 +- 0.5e-5 in every single output, whatever the signs of the inputs.  Therefore the
+// second half of every chunk (words 2 and 3) is staged with the inputs of those sums NEGATED and
+// added up in an accumulator of its own, which is subtracted: the two halves lose the same on
+// average and the bias cancels (the sums of nibble * 2^-20 * x lose 16 times less and are left alone).
+__device__ __forceinline__ u32x4 staged_order(const u32x4 v, int word)
+{
+    const uint32_t flip = word >= 2 ? 0x80008000u : 0u;
+    u32x4 o;
+    o[0] = ((v[0] & 0xFFFFu) | (v[2] << 16)) ^ flip; // x0, x4 (meet the nibbles at bit 0 of a byte)
+    o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u);      // x1, x5
+    o[2] = ((v[1] & 0xFFFFu) | (v[3] << 16)) ^ flip; // x2, x6 (bit 0 of a byte after the shift by 8)
+    o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u);      // x3, x7
+    return o;
+}
+
+// One thread's pieces of the input into the LDS image; `tid` < 256.
 template <int J>
-__device__ __forceinline__ void commit_pieces(u32x4* xs, float* sx, const VecPieces<J>& p)
+__device__ __forceinline__ void commit_pieces_t(u32x4* xs, float* sx, const VecPieces<J>& p, int tid)
 {
     constexpr int JC = J * 64;
 #pragma unroll
     for (int i = 0; i < J; ++i) { // JC*4 pieces over 256 threads = J per thread
-        const int e = threadIdx.x + i * 256;
+        const int e = tid + i * 256;
         const u32x4 v = p.v[i];
-        u32x4 o;
-        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);     // x0,x4
-        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u); // x1,x5
-        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);     // x2,x6
-        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u); // x3,x7
-        xs[(e & 3) * JC + (e >> 2)] = o;
+        xs[(e & 3) * JC + (e >> 2)] = staged_order(v, e & 3);
         const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
         float s = 0.0f;
 #pragma unroll
@@ -121,6 +138,12 @@ __device__ __forceinline__ void commit_pieces(u32x4* xs, float* sx, const VecPie
         if ((e & 3) == 0)
             sx[e >> 2] = s;
     }
+}
+
+template <int J>
+__device__ __forceinline__ void commit_pieces(u32x4* xs, float* sx, const VecPieces<J>& p)
+{
+    commit_pieces_t<J>(xs, sx, p, static_cast<int>(threadIdx.x));
 }
 
 // Dot products of R rows (J chunks per lane each) with the staged input.
@@ -142,18 +165,22 @@ __device__ __forceinline__ void dot_frag(float (&acc)[R], const Frag<J, R>& f, c
         const float sxv = sx[c];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-            float a0 = 0.0f, a1 = 0.0f; // a0: nibbles at bit 0 of a byte (x 2^-24), a1: at bit 4 (x 2^-20)
+            // a0, a0n: nibbles at bit 0 of a byte (x 2^-24) of words 0-1 and, inputs negated, of words 2-3;
+            // a1: nibbles at bit 4 (x 2^-20)
+            float a0 = 0.0f, a0n = 0.0f, a1 = 0.0f;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const uint32_t w = f.w[r][j][i], w8 = w >> 8;
-                a0 = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[i][0]), a0, false);  // n0,n4
+                float& lo = i < 2 ? a0 : a0n;
+                lo = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[i][0]), lo, false);  // n0,n4
                 a1 = __builtin_amdgcn_fdot2(as_h2(w & 0x00F000F0u), as_h2(xv[i][1]), a1, false);  // n1,n5
-                a0 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[i][2]), a0, false); // n2,n6
+                lo = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[i][2]), lo, false); // n2,n6
                 a1 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), as_h2(xv[i][3]), a1, false); // n3,n7
             }
             const float zf = static_cast<float>((f.zw[r][j] >> zshift) & 0xFu);
-            float t = a0 * 16777216.0f;  // 2^24
-            t = fmaf(a1, 1048576.0f, t); // 2^20
+            float t = a0 * 16777216.0f;      // 2^24
+            t = fmaf(a0n, -16777216.0f, t);
+            t = fmaf(a1, 1048576.0f, t);     // 2^20
             t = fmaf(-zf, sxv, t);       // sum x (n - z)
             acc[r] = fmaf(t, half_bits_to_float(f.sb[r][j]), acc[r]);
         }
@@ -399,33 +426,6 @@ __device__ __forceinline__ void expand(Frag<J, R>& f, const CFrag<J, R>& c, int 
             f.sb[r][j] = static_cast<uint16_t>(
                 __builtin_amdgcn_ds_bpermute((((lane >> 2) + 16 * j) & 63) * 4, static_cast<int>(c.sbv[r][j >> 2])));
         }
-}
-
-// commit_pieces for thread `tid` of the first 256 of a larger workgroup.
-template <int J>
-__device__ __forceinline__ void commit_pieces_t(u32x4* xs, float* sx, const VecPieces<J>& p, int tid)
-{
-    constexpr int JC = J * 64;
-#pragma unroll
-    for (int i = 0; i < J; ++i) {
-        const int e = tid + i * 256;
-        const u32x4 v = p.v[i];
-        u32x4 o;
-        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);     // x0,x4
-        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u); // x1,x5
-        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);     // x2,x6
-        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u); // x3,x7
-        xs[(e & 3) * JC + (e >> 2)] = o;
-        const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
-        float s = 0.0f;
-#pragma unroll
-        for (int k = 0; k < 4; ++k)
-            s = __builtin_amdgcn_fdot2(as_h2(v[k]), one, s, false);
-        s += dpp_f32<DPP_QUAD_XOR1>(s);
-        s += dpp_f32<DPP_QUAD_XOR2>(s);
-        if ((e & 3) == 0)
-            sx[e >> 2] = s;
-    }
 }
 
 // Rows per block: what fits in 8 weight loads (32 registers) per item; RB x ss <= 128 scales
@@ -895,12 +895,7 @@ __global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(a.x, a.K * 2);
     for (int e = threadIdx.x; e < nchunks * 4; e += 256) {
         const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(rx, e * 16, 0, 0);
-        u32x4 o;
-        o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);
-        o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u);
-        o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);
-        o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u);
-        xs_dyn[(e & 3) * nchunks + (e >> 2)] = o;
+        xs_dyn[(e & 3) * nchunks + (e >> 2)] = staged_order(v, e & 3);
         const h2_t one = {static_cast<_Float16>(1.0f), static_cast<_Float16>(1.0f)};
         float s = 0.0f;
 #pragma unroll
@@ -930,18 +925,20 @@ __global__ __launch_bounds__(256) void int4_matvec_generic_kernel(Int4Args a)
                 const uint32_t zw = __builtin_amdgcn_raw_buffer_load_b32(rz, (c >> 5) * 4, 0, 0);
                 const uint16_t sb = __builtin_amdgcn_raw_buffer_load_b16(rs, (c >> 2) * 2, 0, 0);
                 const int cc = c < nchunks ? c : nchunks - 1;
-                float a0 = 0.0f, a1 = 0.0f;
+                float a0 = 0.0f, a0n = 0.0f, a1 = 0.0f;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const u32x4 xv = xs_dyn[i * nchunks + cc];
                     const uint32_t w = w4[i], w8 = w >> 8;
-                    a0 = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[0]), a0, false);
+                    float& lo = i < 2 ? a0 : a0n;
+                    lo = __builtin_amdgcn_fdot2(as_h2(w & 0x000F000Fu), as_h2(xv[0]), lo, false);
                     a1 = __builtin_amdgcn_fdot2(as_h2(w & 0x00F000F0u), as_h2(xv[1]), a1, false);
-                    a0 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[2]), a0, false);
+                    lo = __builtin_amdgcn_fdot2(as_h2(w8 & 0x000F000Fu), as_h2(xv[2]), lo, false);
                     a1 = __builtin_amdgcn_fdot2(as_h2(w8 & 0x00F000F0u), as_h2(xv[3]), a1, false);
                 }
                 const float zf = static_cast<float>((zw >> zshift) & 0xFu);
                 float tt = a0 * 16777216.0f;
+                tt = fmaf(a0n, -16777216.0f, tt);
                 tt = fmaf(a1, 1048576.0f, tt);
                 tt = fmaf(-zf, c < nchunks ? sx[cc] : 0.0f, tt);
                 s = fmaf(tt, half_bits_to_float(sb), s);
