@@ -182,6 +182,22 @@ int llama2_vec_mat(llama2_half* output, const llama2_half* vector, const llama2_
                    int rows, int cols, int m_col_stride, int o_stride, int m_row_stride,
                    int n_heads);
 
+/* llama2_vec_mat for callers that cannot allocate (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same
+ * arguments, same kernels, same results bit for bit; but where llama2_vec_mat keeps the fp32
+ * partial sums of a sequence split over workgroups in a buffer it allocates (and grows) on
+ * demand, this entry point keeps them in a fixed array of LLAMA2_STATIC_VEC_MAT_BYTES inside
+ * the library's code object (one copy per GPU, held until the process ends) and calls no
+ * hipMalloc, hipFree or other allocating routine.  A call whose partial sums
+ * (sequence blocks x n_heads x rows floats) do not fit returns LLAMA2_ERR_UNSUPPORTED
+ * (32 heads of 128 rows fit at any sequence length; 40 heads up to about 3300 positions).
+ * All calls on a GPU share the array: calls that overlap on one GPU (two streams, two
+ * replaying graphs) race; calls on the library's one stream are in order and safe. */
+#define LLAMA2_STATIC_VEC_MAT_BYTES 2097152
+int llama2_vec_mat_static(llama2_half* output, const llama2_half* vector, const llama2_half* matrix,
+                   int rows, int cols, int m_col_stride, int o_stride, int m_row_stride,
+                   int n_heads);
+
 /* Transformer.MultiHeadAttention (src/Transformer.cs:150-156) as ONE launch:
  * scores over `seq_length` rows of `key`, softmax, weighted sum of `value`
  * rows, without the round trip through the `attention` scratch.  key / value

@@ -93,6 +93,7 @@ _SIGNATURES = {
     "llama2_mat_vec": [vp, vp, vp, i, i],
     "llama2_mat_vec_strided": [vp, vp, vp, i, i, i, i, i, i, f, i],
     "llama2_vec_mat": [vp, vp, vp, i, i, i, i, i, i],
+    "llama2_vec_mat_static": [vp, vp, vp, i, i, i, i, i, i],
     "llama2_multi_head_attention": [vp, vp, vp, vp, i, i, i, f, i],
     "llama2_rope_multi_head_attention": [vp, vp, vp, vp, i, i, i, f, i, i, f],
     "llama2_rmsnorm": [vp, vp, vp, i, f],

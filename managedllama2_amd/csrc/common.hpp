@@ -48,6 +48,8 @@ Context& ctx();
 int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
 int hip_fail(hipError_t e, const char* what);
 int ensure_attn_partials(size_t bytes);
+// Device address of llama2_vec_mat_static's scratch array on `device` (current), asked for once at llama2_init.
+int resolve_vec_mat_static_scratch(int device);
 // Sampler.Sample's stochastic branch in one launch (sampler.hip).  token_only: the caller reads the
 // token alone, so the sort may stop at the head of the distribution that holds top_p of the mass.
 int sample_launch(const char* fn, uint16_t* logits, int* indices, int size, float temperature, float top_p, float coin,

@@ -352,6 +352,87 @@ static int pick_t_per_wg(int cols, int other_dim_wgs, int min_t)
 
 using namespace l2;
 
+// ---------------------------------------------------------------- static scratch
+// llama2_vec_mat_static allocates nothing: the fp32 partial sums of a sequence split over
+// workgroups live in this file-scope device array (one copy per GPU, at its own address, held
+// until the process ends).  In host code the array's name is only a stand-in; its device address
+// is asked for once per device, at llama2_init with that device current, and every later use
+// goes through that pointer.  Nothing in the array has to start at zero: the first launch writes
+// every partial sum the second one reads.
+static __device__ __align__(256) float scratch[LLAMA2_STATIC_VEC_MAT_BYTES / sizeof(float)];
+
+namespace l2 {
+
+constexpr int kMaxStaticDevices = 64;
+static float* g_static_partials[kMaxStaticDevices] = {};
+
+int resolve_vec_mat_static_scratch(int device)
+{
+    if (device < 0 || device >= kMaxStaticDevices)
+        return fail(LLAMA2_ERR_INVALID_ARGUMENT, "llama2_init: device %d beyond the %d the static scratch tracks", device,
+                    kMaxStaticDevices);
+    void* ptr = nullptr;
+    L2_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr)
+        return fail(LLAMA2_ERR_NO_DEVICE, "llama2_init: the static scratch has no address on device %d", device);
+    g_static_partials[device] = static_cast<float*>(ptr);
+    return LLAMA2_OK;
+}
+
+// VecMat.Forward; `static_partials`: the caller's scratch for the partial sums (LLAMA2_STATIC_VEC_MAT_BYTES of
+// it), or null: the library's growing buffer.
+static int vec_mat(const char* fn, llama2_half* output, const llama2_half* vector, const llama2_half* matrix, int rows,
+                   int cols, int m_col_stride, int o_stride, int m_row_stride, int n_heads, float* static_partials)
+{
+    L2_CHECK(output && vector && matrix, "%s: null pointer", fn);
+    L2_CHECK(rows > 0 && cols > 0 && n_heads > 0, "%s: rows=%d cols=%d n_heads=%d must be positive", fn, rows, cols,
+             n_heads);
+    L2_CHECK(m_col_stride >= 0 && m_row_stride >= 0 && o_stride >= 0, "%s: negative stride", fn);
+    const bool fast =
+        rows % 8 == 0 && m_col_stride % 8 == 0 && m_row_stride % 8 == 0 && aligned(matrix, 16);
+    if (fast && rows == 128 && cols <= kHeadVecMatCols) {
+        hipLaunchKernelGGL(vecmat_head_kernel, dim3(n_heads), dim3(1024), 0, ctx().stream, output, vector, matrix, cols,
+                           m_col_stride, o_stride, m_row_stride);
+        L2_LAUNCH_CHECK(fn);
+    } else if (fast) {
+        const int hq = ceil_div(n_heads, 4), rb = ceil_div(rows, 128);
+        const int t_per_wg = pick_t_per_wg(cols, hq * rb, 32);
+        const int splits = ceil_div(cols, t_per_wg);
+        const dim3 grid(splits, hq, rb);
+        float* partials = nullptr;
+        if (splits > 1) {
+            const size_t bytes = static_cast<size_t>(splits) * n_heads * rows * sizeof(float);
+            if (static_partials) {
+                if (bytes > LLAMA2_STATIC_VEC_MAT_BYTES)
+                    return fail(LLAMA2_ERR_UNSUPPORTED,
+                                "%s: %d sequence blocks x %d heads x %d rows of partial sums (%zu bytes) exceed the static "
+                                "scratch of %d bytes; use llama2_vec_mat", fn, splits, n_heads, rows, bytes,
+                                LLAMA2_STATIC_VEC_MAT_BYTES);
+                partials = static_partials;
+            } else {
+                if (int rc = ensure_attn_partials(bytes))
+                    return rc;
+                partials = ctx().attn_partials;
+            }
+        }
+        hipLaunchKernelGGL((vecmat_kernel<4>), grid, dim3(kThreads), 0, ctx().stream, output, partials, vector,
+                           matrix, rows, cols, m_col_stride, o_stride, m_row_stride, n_heads, t_per_wg);
+        L2_LAUNCH_CHECK(fn);
+        if (splits > 1) {
+            hipLaunchKernelGGL(vecmat_reduce_kernel, dim3(ceil_div(n_heads * rows, 64)), dim3(kReduceWaves * 64), 0,
+                               ctx().stream, output, partials, rows, o_stride, n_heads, splits);
+            L2_LAUNCH_CHECK("vecmat_reduce_kernel");
+        }
+    } else {
+        hipLaunchKernelGGL(vecmat_generic_kernel, dim3(ceil_div(n_heads * rows, 256)), dim3(256), 0, ctx().stream,
+                           output, vector, matrix, rows, cols, m_col_stride, o_stride, m_row_stride, n_heads);
+        L2_LAUNCH_CHECK(fn);
+    }
+    return LLAMA2_OK;
+}
+
+} // namespace l2
+
 extern "C" {
 
 int llama2_mat_vec(llama2_half* output, const llama2_half* vector, const llama2_half* matrix, int rows, int cols)
@@ -407,42 +488,21 @@ int llama2_vec_mat(llama2_half* output, const llama2_half* vector, const llama2_
                    int m_col_stride, int o_stride, int m_row_stride, int n_heads)
 {
     L2_REQUIRE_INIT();
-    const char* fn = "llama2_vec_mat";
-    L2_CHECK(output && vector && matrix, "%s: null pointer", fn);
-    L2_CHECK(rows > 0 && cols > 0 && n_heads > 0, "%s: rows=%d cols=%d n_heads=%d must be positive", fn, rows, cols,
-             n_heads);
-    L2_CHECK(m_col_stride >= 0 && m_row_stride >= 0 && o_stride >= 0, "%s: negative stride", fn);
-    const bool fast =
-        rows % 8 == 0 && m_col_stride % 8 == 0 && m_row_stride % 8 == 0 && aligned(matrix, 16);
-    if (fast && rows == 128 && cols <= kHeadVecMatCols) {
-        hipLaunchKernelGGL(vecmat_head_kernel, dim3(n_heads), dim3(1024), 0, ctx().stream, output, vector, matrix, cols,
-                           m_col_stride, o_stride, m_row_stride);
-        L2_LAUNCH_CHECK(fn);
-    } else if (fast) {
-        const int hq = ceil_div(n_heads, 4), rb = ceil_div(rows, 128);
-        const int t_per_wg = pick_t_per_wg(cols, hq * rb, 32);
-        const int splits = ceil_div(cols, t_per_wg);
-        const dim3 grid(splits, hq, rb);
-        float* partials = nullptr;
-        if (splits > 1) {
-            if (int rc = ensure_attn_partials(static_cast<size_t>(splits) * n_heads * rows * sizeof(float)))
-                return rc;
-            partials = ctx().attn_partials;
-        }
-        hipLaunchKernelGGL((vecmat_kernel<4>), grid, dim3(kThreads), 0, ctx().stream, output, partials, vector,
-                           matrix, rows, cols, m_col_stride, o_stride, m_row_stride, n_heads, t_per_wg);
-        L2_LAUNCH_CHECK(fn);
-        if (splits > 1) {
-            hipLaunchKernelGGL(vecmat_reduce_kernel, dim3(ceil_div(n_heads * rows, 64)), dim3(kReduceWaves * 64), 0,
-                               ctx().stream, output, partials, rows, o_stride, n_heads, splits);
-            L2_LAUNCH_CHECK("vecmat_reduce_kernel");
-        }
-    } else {
-        hipLaunchKernelGGL(vecmat_generic_kernel, dim3(ceil_div(n_heads * rows, 256)), dim3(256), 0, ctx().stream,
-                           output, vector, matrix, rows, cols, m_col_stride, o_stride, m_row_stride, n_heads);
-        L2_LAUNCH_CHECK(fn);
-    }
-    return LLAMA2_OK;
+    return vec_mat("llama2_vec_mat", output, vector, matrix, rows, cols, m_col_stride, o_stride, m_row_stride, n_heads,
+                   nullptr);
+}
+
+int llama2_vec_mat_static(llama2_half* output, const llama2_half* vector, const llama2_half* matrix, int rows, int cols,
+                          int m_col_stride, int o_stride, int m_row_stride, int n_heads)
+{
+    L2_REQUIRE_INIT();
+    const char* fn = "llama2_vec_mat_static";
+    const int device = ctx().device;
+    float* sp = device >= 0 && device < kMaxStaticDevices ? g_static_partials[device] : nullptr;
+    if (!sp)
+        return fail(LLAMA2_ERR_NOT_INITIALIZED, "%s: the static scratch of device %d was not resolved at llama2_init", fn,
+                    device);
+    return vec_mat(fn, output, vector, matrix, rows, cols, m_col_stride, o_stride, m_row_stride, n_heads, sp);
 }
 
 } // extern "C"

@@ -109,6 +109,10 @@ int llama2_init(int device)
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_keys), LLAMA2_MAX_SAMPLER_SIZE * sizeof(uint16_t)));
     L2_HIP(hipMalloc(reinterpret_cast<void**>(&c.sort_values), LLAMA2_MAX_SAMPLER_SIZE * sizeof(int)));
     c.device = device;
+    if (int rc = resolve_vec_mat_static_scratch(device)) {
+        c.device = -1;
+        return rc;
+    }
     c.int4_narrow = getenv("LLAMA2_INT4_NARROW") != nullptr;
     c.int4_blocks = getenv("LLAMA2_INT4_BLOCKS") != nullptr;
     c.int4_no_span = getenv("LLAMA2_INT4_NO_SPAN") != nullptr;
