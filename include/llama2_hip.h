@@ -381,8 +381,9 @@ typedef struct llama2_decoder llama2_decoder;
  * (src/Transformer.cs:158-190) as ONE persistent launch -- one workgroup per
  * compute unit walks through all layers, the vectors between the modules are
  * handed from workgroup to workgroup inside the launch, and the weight stream
- * never stops at a module boundary.  Same arithmetic, same results as
- * LLAMA2_DECODE_FUSED.  Serves histories of up to 3072 rows (longer ones fall
+ * never stops at a module boundary.  Same arithmetic as LLAMA2_DECODE_FUSED, and
+ * the same results bit for bit up to 1024 attended rows (beyond, the launch
+ * sequence merges attention blocks of 256 rows and this step blocks of 128).  Serves histories of up to 3072 rows (longer ones fall
  * back to the launch sequence, step by step) and the shapes it has kernels for
  * (Llama-2-7B: dim 4096, hidden_dim 11008, 32 heads on 256 compute units; and
  * small models of at most one row per wavefront and phase: on 256 compute units

@@ -28,6 +28,7 @@ struct Context {
     bool int4_narrow = false;
     bool int4_blocks = false;
     bool int4_no_span = false;
+    int attn_waves = 0; // LLAMA2_ATTN_WAVES: block size of the attention entry points, for sweeps (0: by length)
     // fp32 partial sums of the sequence-split attention kernels
     float* attn_partials = nullptr;
     size_t attn_partials_bytes = 0;

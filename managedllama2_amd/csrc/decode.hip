@@ -38,43 +38,58 @@ namespace l2 {
 // One compute unit pulls only a few tens of GB/s, so a short sequence wants
 // many small blocks (4 wavefronts, 128 rows); the exchange between workgroups
 // costs about 3 us whatever their number, and a long sequence wants fewer
-// merges (16 wavefronts, 512 rows).  Dispatching workgroups that find nothing
-// to do is not free: a grid sized for the whole context costs several
-// microseconds per launch at short lengths.  The position lives on the device,
-// but the host always knows an upper bound for it, so it picks the launch
-// shape (block size, number of blocks) from a short list by that bound.
+// merges.  Measured on 32 heads (one launch, RoPE inside), 64 / 128 / 256 / 512
+// rows per block: 512 rows 7.4 / 7.3 / 8.8 / 11.0 us, 2048 rows 17.7 / 12.1 /
+// 11.4 / 15.5 us, 4096 rows 31.2 / 21.5 / 17.3 / 19.4 us: 128-row blocks up to
+// 1024 rows, 256-row blocks (8 wavefronts) beyond.  Dispatching workgroups
+// that find nothing to do is not free: a grid sized for the whole context costs
+// several microseconds per launch at short lengths.  The position lives on the
+// device, but the host always knows an upper bound for it, so it picks the
+// launch shape (block size, number of blocks) from a short list by that bound.
 // Measured in the decode loop: one 256-row block of 8 wavefronts for 129 .. 256 rows
 // is as fast as two 128-row blocks and a merge, two 256-row blocks for 257 .. 512 rows
 // lose 1.2 % against four 128-row blocks.
 constexpr int kAttnWaves = 16;
-constexpr int kSplitT = 32 * kAttnWaves; // 512
+constexpr int kSplitT = 32 * kAttnWaves; // 512: only for contexts beyond 64 blocks of 256 rows
+constexpr int kMidWaves = 8;
+constexpr int kMidSplitT = 32 * kMidWaves; // 256
 constexpr int kSmallWaves = 4;
 constexpr int kSmallSplitT = 32 * kSmallWaves; // 128
 constexpr int kMaxSplits = 64; // one lane per block in the merge
 constexpr int kPartStride = kRopeHeadSize + 2; // 128 partial outputs, block max, block sum
 
 inline int attn_max_splits(int seq_len) { return ceil_div(seq_len, kSplitT); }
-constexpr int kSmallBlockMaxSeq = 3072; // 128-row blocks up to this length, 512-row blocks beyond
+constexpr int kSmallBlockMaxSeq = 1024;                   // 128-row blocks up to this length,
+constexpr int kMidBlockMaxSeq = kMaxSplits * kMidSplitT;  // 256-row blocks up to this one (16384), 512-row blocks beyond
 
-// Launch shapes of the decode step: index b < kAttnShapes - 1 is 2^b blocks of 128
-// rows, the last index is 512-row blocks over the whole context.
+// Launch shapes of the decode step: 1, 2, 4, 8 blocks of 128 rows; 8, 16, 32, 64 blocks
+// of 256 rows; 512-row blocks over the whole context.
 constexpr int ceil_log2(int v) { return v <= 1 ? 0 : 1 + ceil_log2((v + 1) / 2); }
-constexpr int kAttnShapes = ceil_log2(kSmallBlockMaxSeq / kSmallSplitT) + 2;
+constexpr int kSmallShapes = ceil_log2(kSmallBlockMaxSeq / kSmallSplitT) + 1;             // 4
+constexpr int kMidFirstLog = ceil_log2(kSmallBlockMaxSeq / kMidSplitT) + 1;               // 3: 8 blocks
+constexpr int kMidShapes = ceil_log2(kMaxSplits) - kMidFirstLog + 1;                      // 4
+constexpr int kAttnShapes = kSmallShapes + kMidShapes + 1;
 struct AttnShape {
     int waves;
     int splits;
 };
 inline int attn_shape_index(int rows)
 {
-    if (rows > kSmallBlockMaxSeq)
-        return kAttnShapes - 1;
-    return ceil_log2(ceil_div(rows, kSmallSplitT));
+    if (rows <= kSmallBlockMaxSeq)
+        return ceil_log2(ceil_div(rows, kSmallSplitT));
+    if (rows <= kMidBlockMaxSeq) {
+        const int b = ceil_log2(ceil_div(rows, kMidSplitT));
+        return kSmallShapes + (b > kMidFirstLog ? b - kMidFirstLog : 0);
+    }
+    return kAttnShapes - 1;
 }
 inline AttnShape attn_shape(int index, int seq_len)
 {
-    if (index == kAttnShapes - 1)
-        return AttnShape{kAttnWaves, attn_max_splits(seq_len)};
-    return AttnShape{kSmallWaves, 1 << index};
+    if (index < kSmallShapes)
+        return AttnShape{kSmallWaves, 1 << index};
+    if (index < kSmallShapes + kMidShapes)
+        return AttnShape{kMidWaves, 1 << (kMidFirstLog + index - kSmallShapes)};
+    return AttnShape{kAttnWaves, attn_max_splits(seq_len)};
 }
 
 struct AttnArgs;
@@ -310,20 +325,24 @@ __global__ __launch_bounds__(WAVES * 64) void fused_attn_kernel(AttnArgs a)
     }
 }
 
+template <int WAVES>
+static void launch_attn_waves(const dim3 grid, const AttnArgs& a)
+{
+    if (a.q_rw)
+        hipLaunchKernelGGL((fused_attn_kernel<WAVES, true>), grid, dim3(WAVES * 64), 0, ctx().stream, a);
+    else
+        hipLaunchKernelGGL((fused_attn_kernel<WAVES, false>), grid, dim3(WAVES * 64), 0, ctx().stream, a);
+}
+
 void launch_attn(const AttnShape& shape, int n_heads, const AttnArgs& a)
 {
-    const dim3 grid(shape.splits, n_heads), block(shape.waves * 64);
-    if (a.q_rw) {
-        if (shape.waves == kSmallWaves)
-            hipLaunchKernelGGL((fused_attn_kernel<kSmallWaves, true>), grid, block, 0, ctx().stream, a);
-        else
-            hipLaunchKernelGGL((fused_attn_kernel<kAttnWaves, true>), grid, block, 0, ctx().stream, a);
-        return;
+    const dim3 grid(shape.splits, n_heads);
+    switch (shape.waves) {
+    case 2: launch_attn_waves<2>(grid, a); break;
+    case 4: launch_attn_waves<4>(grid, a); break;
+    case 8: launch_attn_waves<8>(grid, a); break;
+    default: launch_attn_waves<kAttnWaves>(grid, a); break;
     }
-    if (shape.waves == kSmallWaves)
-        hipLaunchKernelGGL((fused_attn_kernel<kSmallWaves, false>), grid, block, 0, ctx().stream, a);
-    else
-        hipLaunchKernelGGL((fused_attn_kernel<kAttnWaves, false>), grid, block, 0, ctx().stream, a);
 }
 
 // ---------------------------------------------------------------- step state
@@ -781,6 +800,9 @@ int check_attention(const char* fn, const void* output, const void* query, const
              "%s: seq_length * dim = %lld is too large", fn, static_cast<long long>(seq_length) * dim);
     L2_CHECK(seq_length <= kMaxSplits * kSplitT, "%s: seq_length=%d exceeds %d", fn, seq_length, kMaxSplits * kSplitT);
     *shape = attn_shape(attn_shape_index(seq_length), seq_length);
+    const int forced = ctx().attn_waves; // LLAMA2_ATTN_WAVES: 2, 4, 8 or 16 wavefronts (64 .. 512 rows) per block
+    if ((forced == 2 || forced == 4 || forced == 8 || forced == 16) && ceil_div(seq_length, forced * 32) <= kMaxSplits)
+        shape->waves = forced;
     shape->splits = ceil_div(seq_length, shape->waves * 32);
     return LLAMA2_OK;
 }

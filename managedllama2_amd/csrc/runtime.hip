@@ -116,6 +116,7 @@ int llama2_init(int device)
     c.int4_narrow = getenv("LLAMA2_INT4_NARROW") != nullptr;
     c.int4_blocks = getenv("LLAMA2_INT4_BLOCKS") != nullptr;
     c.int4_no_span = getenv("LLAMA2_INT4_NO_SPAN") != nullptr;
+    c.attn_waves = getenv("LLAMA2_ATTN_WAVES") ? atoi(getenv("LLAMA2_ATTN_WAVES")) : 0;
     c.ready = true;
     g_err[0] = 0;
     return LLAMA2_OK;

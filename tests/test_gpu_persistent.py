@@ -69,8 +69,11 @@ def test_persistent_equals_fused_bit_for_bit():
 
 @pytest.mark.parametrize("pos", [127, 128, 511, 512, 1100, 3071, 3072, 3100])
 def test_persistent_step_with_long_history(oracle, pos):
-    """1, 2, 4, 5, 9 and 24 attention blocks; from 3072 rows on the decoder falls
-    back to the launch sequence for the step."""
+    """1, 2, 4, 5, 9 and 24 attention blocks of 128 rows; from 3072 rows on the decoder falls
+    back to the launch sequence for the step.  Up to 1024 attended rows the launch sequence uses
+    128-row blocks as well and the two agree bit for bit; beyond, the launch sequence merges
+    256-row blocks (a different, equally valid grouping of the same sums), and the comparison is
+    norm-wise at the per-module tolerance."""
     cfg = dict(HS128, seq_len=max(1200, pos + 40))
     dim, L, S = cfg["dim"], cfg["n_layers"], cfg["seq_len"]
     model = synth.random_model(cfg, seed=11, rms_random=True)
@@ -90,9 +93,15 @@ def test_persistent_step_with_long_history(oracle, pos):
         vrow = t.runstate.valueCache.to_host(dim, (L - 1) * S * dim + pos * dim)
         outs.append((t.runstate.logits.to_host(), row, vrow))
         t.close()
-    for other in outs[1:]:
-        for a, b, what in zip(outs[0], other, ("logits", "k row", "v row")):
+    same_blocks = pos + 1 <= 1024 or pos + 1 > 3072
+    for a, b, what in zip(outs[1], outs[2], ("logits", "k row", "v row")):  # persistent: eager == graph replay
+        assert np.array_equal(bits(a), bits(b)), "%s at pos %d" % (what, pos)
+    for a, b, what in zip(outs[0], outs[1], ("logits", "k row", "v row")):
+        if same_blocks:
             assert np.array_equal(bits(a), bits(b)), "%s at pos %d" % (what, pos)
+        else:
+            err = np.max(np.abs(a.astype(np.float64) - b.astype(np.float64))) / np.max(np.abs(a.astype(np.float64)))
+            assert err <= 2e-3, "%s at pos %d: %.2e" % (what, pos, err)
     if pos in (128, 3071):
         hm = oracle.HostModel(cfg, model)
         hm.key_cache[:], hm.value_cache[:] = kc, vc

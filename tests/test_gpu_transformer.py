@@ -108,10 +108,10 @@ def test_fused_step_tracks_module_step(oracle):
     assert_close_normwise(outs[1][1].astype(np.float64), outs[0][1].astype(np.float64), "fused vs modules K cache", 2e-3)
 
 
-@pytest.mark.parametrize("pos", [127, 128, 511, 512, 1100, 3071, 3072])
+@pytest.mark.parametrize("pos", [127, 128, 511, 512, 1023, 1024, 2047, 2048, 3072])
 def test_fused_step_with_long_history(oracle, pos):
-    """A step whose history spans 1, 2, 4, 5, 9 and 24 blocks of 128 rows and 7
-    blocks of 512 rows (the attention launch shapes either side of each change):
+    """A step whose history spans 1, 2, 4, 5 and 8 blocks of 128 rows and 5, 8, 9 and 13
+    blocks of 256 rows (the attention launch shapes either side of each change):
     the caches are filled with random rows, then one step of the module
     sequence, the fused launches, the graph replay and the oracle are compared."""
     cfg = dict(HS128, seq_len=max(1200, pos + 40))
