@@ -490,10 +490,11 @@ def main():
         far_ms = ev.stop_ms()
         result["decode"]["tokens_per_s_at_position_%d" % far] = round(64 / (far_ms * 1e-3), 1)
         log("decode at positions %d..%d: %.1f tok/s" % (far, far + 63, 64 / (far_ms * 1e-3)))
-        # the reference's own loop shape (Transformer.Generate: forward, sample, read the token back on the
-        # host every step) over the same launches: what a host that keeps its loop gets
+        # the reference's own loop shape (Transformer.Generate: forward every step, sample and read the token
+        # back on the host for every generated token) over the same positions and launches: what a host that
+        # keeps its loop gets
         t1 = time.perf_counter()
-        n_host = sum(1 for _ in model.Generate(prompt, 192, stop_on_special=False))
+        n_host = sum(1 for _ in model.Generate(prompt, steps, stop_on_special=False))
         host_tok_s = n_host / (time.perf_counter() - t1)
         result["decode"]["host_loop_tokens_per_s"] = round(host_tok_s, 1)
         log("decode, host loop with one read-back per token: %.1f tok/s" % host_tok_s)
@@ -548,7 +549,7 @@ def main():
             sp, coins = model.sampler, np.random.default_rng(7)
             sp.temperature, sp.topP, sp.random = temp, top_p, coins.random
             t1 = time.perf_counter()
-            n_host = sum(1 for _ in model.Generate(prompt, 192, stop_on_special=False))
+            n_host = sum(1 for _ in model.Generate(prompt, steps, stop_on_special=False))
             sampler["host_loop_tokens_per_s"] = round(n_host / (time.perf_counter() - t1), 1)
             sp.temperature = 0.0
         result["sampler"] = sampler

@@ -733,7 +733,18 @@ __global__ __launch_bounds__(WAVES * 64) void int4_matvec_span_kernel(Int4Args a
             w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
     };
 
-    // input first, then the span's scales / zero words / residuals, then the first row
+    // The position of the step, for the cache row of k and v: requested ahead of everything else as a
+    // vector load and taken into a scalar register only where it is used.  Vector loads return in order
+    // and are waited for by count; read where it is used (`a.pos_ptr[0]` after the first row's requests)
+    // it made the wavefront wait for that whole row before the input could be staged.
+    uint32_t pos_bits = 0;
+    if (MODE == QKV_ROPE)
+        pos_bits = __builtin_amdgcn_raw_buffer_load_b32(make_rsrc(a.pos_ptr, a.pos_ptr ? 4 : 0), 0, 0, 0);
+    auto position = [&]() -> int {
+        asm volatile("" : "+v"(pos_bits)); // stays where it is written
+        return __builtin_amdgcn_readfirstlane(static_cast<int>(pos_bits)); // 0 without pos_ptr: nothing was read
+    };
+    // input next, then the span's scales / zero words / residuals, then the first row
     const bool stager = WAVES == 4 || threadIdx.x < 256;
     VecPieces<J> xp, gp;
     const uint16_t* xsrc = a.x;
@@ -769,16 +780,18 @@ __global__ __launch_bounds__(WAVES * 64) void int4_matvec_span_kernel(Int4Args a
     load_w(ring[0], 0);
     asm volatile("" ::: "memory");
 
-    const int pos = MODE == QKV_ROPE && a.pos_ptr ? a.pos_ptr[0] : 0;
     if (MODE == QKV_ROPE) {
         if (a.rope_table) { // prepared by the kernel that set the position
             if (threadIdx.x < kRopeHeadSize)
                 rope_tab[threadIdx.x] = rope_entry;
-        } else if (threadIdx.x < kRopeHeadSize / 2) {
-            float c, sn;
-            rope_cos_sin(c, sn, threadIdx.x, kRopeHeadSize, pos, a.theta);
-            rope_tab[2 * threadIdx.x] = c;
-            rope_tab[2 * threadIdx.x + 1] = sn;
+        } else {
+            const int pos = position(); // all threads: the value is moved from lane 0
+            if (threadIdx.x < kRopeHeadSize / 2) {
+                float c, sn;
+                rope_cos_sin(c, sn, threadIdx.x, kRopeHeadSize, pos, a.theta);
+                rope_tab[2 * threadIdx.x] = c;
+                rope_tab[2 * threadIdx.x + 1] = sn;
+            }
         }
     }
     if (STAGE == STAGE_RMSNORM) {
@@ -845,6 +858,7 @@ __global__ __launch_bounds__(WAVES * 64) void int4_matvec_span_kernel(Int4Args a
             pair_val[2 * wave + 1] = kv;
         }
         __syncthreads();
+        const int pos = position();
         if (lane == 0 && n) {
             const int partner = wave ^ 4, i = r0 & 63; // pair index within the head
             const float c = rope_tab[2 * i], sn = rope_tab[2 * i + 1];
