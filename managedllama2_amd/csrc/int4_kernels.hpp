@@ -733,6 +733,20 @@ __global__ __launch_bounds__(WAVES * 64) void int4_matvec_span_kernel(Int4Args a
             w[j] = __builtin_amdgcn_raw_buffer_load_b128(rw, lane * 16 + j * 1024, 0, kAuxStream);
     };
 
+    // The decode step's kernels (RMSNorm in the staging) fetch every kernel argument they read in one
+    // round trip: left to itself the compiler fetches them where they are first used, five dependent
+    // round trips to the scalar cache before the first weight is requested (decode 910 -> 917 tok/s).
+    // The kernels that stage the input as given have shorter chains and lose 1 .. 3 % with it.
+    if (STAGE == STAGE_RMSNORM) {
+        asm volatile("" ::"s"(a.m[0].w), "s"(a.m[0].z), "s"(a.m[0].s), "s"(a.out[0]), "s"(a.x), "s"(a.K), "s"(a.N),
+                     "s"(a.ws), "s"(a.ss), "s"(a.zs), "s"(a.gamma), "s"(a.eps), "s"(a.embedding));
+        if (TN > 1)
+            asm volatile("" ::"s"(a.m[1].w), "s"(a.m[1].z), "s"(a.m[1].s), "s"(a.out[1]));
+        if (TN > 2)
+            asm volatile("" ::"s"(a.m[2].w), "s"(a.m[2].z), "s"(a.m[2].s), "s"(a.out[2]));
+        if (MODE == QKV_ROPE)
+            asm volatile("" ::"s"(a.pos_ptr), "s"(a.kv_dim), "s"(a.rope_table));
+    }
     // The position of the step, for the cache row of k and v: requested ahead of everything else as a
     // vector load and taken into a scalar register only where it is used.  Vector loads return in order
     // and are waited for by count; read where it is used (`a.pos_ptr[0]` after the first row's requests)
