@@ -39,7 +39,7 @@ sys.path.insert(0, ROOT)
 # kernel's source: when csrc/int4_kernels.hpp no longer hashes to the value below, the kernel has changed
 # since the counters were read and `roofline.traffic` is reported as null until they are read again.
 SWIGLU_HBM_TRAFFIC_BYTES = 47048947
-SWIGLU_HBM_TRAFFIC_SOURCE_SHA16 = "2a54346e588d5ed4"
+SWIGLU_HBM_TRAFFIC_SOURCE_SHA16 = "c7112bb214b4b729"
 MIN_REPLAYS = 100   # graph replays behind every headline figure
 MIN_SAMPLES = 50    # replays timed one by one for the spread
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E

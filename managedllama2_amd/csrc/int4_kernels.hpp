@@ -8,8 +8,11 @@
 //     instruction, lane l taking chunks l, l+64, ... (buffer_load_dwordx4
 //     through a per-row buffer resource, so the ragged end of a row reads as
 //     zero without any lane predication);
-//   * wavefronts are persistent: each walks over its rows with the next row's
-//     loads already in flight while the current one is reduced;
+//   * a wavefront owns a span of consecutive rows, all wavefronts resident at once, the row
+//     sequence fully unrolled with the next row's loads in flight while the current one is
+//     reduced (int4_matvec_span_kernel: every shape the decoder and the benches launch); the
+//     two older kernels (persistent wavefronts that stride over the rows, one row or a block of
+//     rows per item) take the launches it refuses;
 //   * the input vector is staged once per workgroup in LDS, pre-permuted to
 //     the order the nibble extraction produces, in four planes so that
 //     consecutive lanes read consecutive 16-byte slots (conflict-free
@@ -677,7 +680,11 @@ __global__ __launch_bounds__(256) void int4_matvec_block_kernel(Int4Args a)
 //     waits for the first weights either;
 //   * results stay in lanes (row i of the span in lane i) and are stored once, after the last row;
 //     residual add and SwiGLU run lane-parallel there;
-//   * the first row of a span is found without a division (base / remainder from the host).
+//   * the first row of a span is found without a division (base / remainder from the host);
+//   * what the instruction stream showed, once read: a load of the position placed after the first
+//     row's requests had become "vector load, wait for everything"; the kernel arguments were
+//     fetched in five dependent round trips; with one row per wavefront the compiler mixed the dot
+//     product into the staging code.  See the comments at those three places below.
 // QKV_ROPE: a workgroup of 8 wavefronts takes rows n .. n + 3 and n + 64 .. n + 67 of a head (of
 // q, k and v), the two halves of four RoPE pairs, and exchanges the fp16-rounded results through LDS.
 // ---------------------------------------------------------------------------------------------
